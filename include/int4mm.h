@@ -1,0 +1,151 @@
+/*
+ * int4mm.h -- C ABI of libint4mm_hip.so: quantized int{4,3,2} x fp16 matvec and
+ * matmul for AMD MI355X (gfx950), plus the pack / unpack helpers of the same
+ * formats.
+ *
+ * Plain pointers and sizes only; no torch types.  Every pointer is a DEVICE
+ * pointer unless stated otherwise.  `stream` is a hipStream_t passed as void*
+ * (NULL = the null stream).  All launches are asynchronous on `stream`; the
+ * functions validate their arguments on the host first and return a non-zero
+ * INT4MM_ERR_* code without launching anything if a check fails.
+ *
+ * Citations name the reference interface each entry point replaces
+ * (paths relative to the mstnegate/int4matmul_kernels checkout).
+ *
+ * Dimension names: K = in_size (reduction dim, unpacked weight rows),
+ * S = out_size (output columns), R = packed rows of `matrix`,
+ * G = rows of scales/zeros, g = group_size.
+ *
+ * Formats (bit-exact with the reference):
+ *   matrix, dense int4/int2 : int32 [K*bits/32, S]; code k of a word at bits
+ *                             bits*(k mod 32/bits), LSB first.
+ *   matrix, dense int3      : int32 [3K/32, S]; every 32 codes of a column are
+ *                             a 96-bit LSB-first stream over 3 rows.
+ *   matrix + mask, 16:32    : mask int32 [K/32, S], bit t of [b,s] set <=> row
+ *                             32b+t kept; matrix int32 [K/16, S], rows 2b,2b+1 =
+ *                             low/high half of the 64-bit word of kept codes in
+ *                             ascending row order, 4 bits each.  Dropped rows
+ *                             decode to exactly 0.
+ *   scales, zeros           : fp16 [G, S], entry (k / g, s), dense k index.
+ *                             scale >= 0: w = fp16(fp16(q - z) * s);
+ *                             scale <  0: w = fp16_fma(+-2^(q & (2^(bits-1)-1)), -s, z),
+ *                             sign = top bit of the code.
+ *   multiplier, outs        : fp16 [B, M, K] and [B, M, S], contiguous.
+ */
+#ifndef INT4MM_H
+#define INT4MM_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#if defined(__GNUC__)
+#define INT4MM_API __attribute__((visibility("default")))
+#else
+#define INT4MM_API
+#endif
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define INT4MM_OK               0
+#define INT4MM_ERR_BITS         1   /* bits not in {4,3,2}          (int4matmul.cpp:35,45)           */
+#define INT4MM_ERR_SPARSE_BITS  2   /* 16:32 mask with bits != 4    (matmul.cuh:184-190,328-332)     */
+#define INT4MM_ERR_SHAPE        3   /* a size rule below is violated (matmul_kernel.cu:379-416)      */
+#define INT4MM_ERR_GROUP        4   /* group_size not a positive multiple of 64 and not negative     */
+#define INT4MM_ERR_NULL         5   /* a required pointer is NULL                                     */
+#define INT4MM_ERR_WORKSPACE    6   /* workspace missing or smaller than int4mm_workspace_bytes()    */
+#define INT4MM_ERR_LAUNCH       7   /* the HIP runtime refused the launch; see int4mm_last_hip_error */
+#define INT4MM_ERR_ALIGN        8   /* a pointer is not 16-byte aligned                              */
+
+/* Human-readable text for a code above (host pointer, static storage). */
+INT4MM_API const char* int4mm_error_string(int code);
+/* hipError_t value of the most recent INT4MM_ERR_LAUNCH on this thread. */
+INT4MM_API int int4mm_last_hip_error(void);
+/* ABI version of this header; bumped on any signature change. */
+INT4MM_API int int4mm_abi_version(void);
+
+/* Benchmark / tuning hook, not part of the drop-in boundary: overrides a launch
+ * heuristic process-wide (value 0 restores the default).  key 0 = matvec waves
+ * per workgroup, 1 = matvec 64-row units per wave, 3 = matmul kernel variant. */
+INT4MM_API int int4mm_tune(int key, int64_t value);
+
+/* Shape of one product.  matrix_rows = R, n_groups = G (rows of scales/zeros).
+ * Rules (violations -> INT4MM_ERR_SHAPE), a strict superset of the reference's
+ * asserts at matmul_kernel.cu:379-416,435-439 and matvec_kernel.cu:307-337,356-360:
+ *   dense : R * 32 == K * bits         sparse (bits == 4) : R * 16 == K
+ *   K % 64 == 0, S % 64 == 0 (README.md:9), B, M >= 1 (B*M*S == 0 returns OK)
+ *   group_size < 0 (one group) or group_size % 64 == 0; g * G >= K
+ */
+typedef struct int4mm_shape {
+    int64_t batch;        /* B */
+    int64_t seq_len;      /* M */
+    int64_t in_size;      /* K */
+    int64_t out_size;     /* S */
+    int64_t matrix_rows;  /* R */
+    int64_t n_groups;     /* G */
+    int64_t group_size;   /* g, or negative for a single group */
+} int4mm_shape;
+
+/* Bytes of device scratch the two products may use for any shape with
+ * out_size <= `max_out_size` (partial sums and arrival counters of the split-K
+ * finish).  The buffer must be zero-filled once before its first use (e.g. with
+ * int4mm_workspace_init); the kernels leave it zeroed where it must be zero.
+ * Calls that share one workspace must not overlap in time. */
+INT4MM_API size_t int4mm_workspace_bytes(int64_t max_out_size);
+INT4MM_API int int4mm_workspace_init(void* workspace, size_t workspace_bytes, void* stream);
+
+/* Matrix-vector product, M == 1 per batch entry:
+ *     outs[b,0,:] = fp16( fp32(outs[b,0,:]) + multiplier[b,0,:] @ W )
+ * i.e. the result is ADDED onto the prior contents of outs, as the reference's
+ * launcher does through its fp32 temporary.
+ * Replaces matvec_packed_int<bits> / matvec_int{4,3,2}
+ * (matvec_kernel.cu:302-387).  shape->seq_len must be 1 (matvec_kernel.cu:323).
+ * sparse_mask == NULL selects the dense format. */
+INT4MM_API int int4mm_matvec(int bits, void* outs, const void* matrix, const void* multiplier,
+                  const void* scales, const void* zeros, const void* sparse_mask,
+                  const int4mm_shape* shape, void* workspace, size_t workspace_bytes,
+                  void* stream);
+
+/* Matrix-matrix product:
+ *     outs[b,m,:] = fp16( sum_k fp32(multiplier[b,m,k]) * fp32(W[k,:]) )   (overwrites outs)
+ * Replaces matmul_packed_int<bits> / matmul_int{4,3,2}
+ * (matmul_kernel.cu:375-463).  Any M >= 1 is accepted. */
+INT4MM_API int int4mm_matmul(int bits, void* outs, const void* matrix, const void* multiplier,
+                  const void* scales, const void* zeros, const void* sparse_mask,
+                  const int4mm_shape* shape, void* workspace, size_t workspace_bytes,
+                  void* stream);
+
+/* 16:32 sparse int4 packer.  wt_in / msk_in: uint8 [S, K] (row = output column;
+ * msk_in > 0 keeps the row); wt_outs: int32 [K/16, S]; msk_outs: int32 [K/32, S].
+ * Requires K % 32 == 0.  Replaces sparse_int4_pack / weight_matrix_packing
+ * (utils_kernel.cu:19-119, int4matmul.cpp:50-63).
+ * bad_blocks (device int32[1], may be NULL) is incremented once for every
+ * (column, 32-row block) whose mask does not keep exactly 16 rows -- the
+ * condition the reference asserts on the device (utils_kernel.cu:41). */
+INT4MM_API int int4mm_sparse_pack(void* wt_outs, void* msk_outs, const void* wt_in, const void* msk_in,
+                       int64_t out_size, int64_t in_size, void* bad_blocks, void* stream);
+
+/* Dense packer for int4/int3/int2: codes uint8 [K, S] (row = k) -> matrix
+ * int32 [K*bits/32, S].  The reference packs dense weights with Python loops
+ * (kernel_test.py:60-123); this is the on-device equivalent of those loops. */
+INT4MM_API int int4mm_dense_pack(int bits, void* matrix_out, const void* codes_in,
+                      int64_t in_size, int64_t out_size, void* stream);
+
+/* Unpack to raw codes: codes_out uint8 [K, S]; keep_out uint8 [K, S] or NULL
+ * (1 = kept; all ones for dense).  Inverse of the two packers; the decode step
+ * of smem_unpack_weights (matmul.cuh:246-405) without the dequantisation. */
+INT4MM_API int int4mm_unpack(int bits, void* codes_out, void* keep_out, const void* matrix,
+                  const void* sparse_mask, int64_t in_size, int64_t out_size, void* stream);
+
+/* Unpack + dequantise to the fp16 matrix the kernels multiply by:
+ * w_out fp16 [K, S], bit-exact with dequantize<> / smem_unpack_weights
+ * (matmul.cuh:115-136,246-428), dropped sparse rows = +0.0. */
+INT4MM_API int int4mm_dequantize(int bits, void* w_out, const void* matrix, const void* scales,
+                      const void* zeros, const void* sparse_mask, int64_t in_size,
+                      int64_t out_size, int64_t n_groups, int64_t group_size, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* INT4MM_H */

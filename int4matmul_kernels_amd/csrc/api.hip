@@ -1,0 +1,112 @@
+// Host-side plumbing of the C ABI: error text, argument validation shared by
+// the two products, tuning knobs and workspace set-up.
+#include "common.h"
+
+#include <atomic>
+
+namespace i4 {
+
+static thread_local int g_last_hip_error = 0;
+static std::atomic<int64_t> g_tuning[TUNE_COUNT];
+
+int check_launch(const char*) {
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        g_last_hip_error = (int)e;
+        return INT4MM_ERR_LAUNCH;
+    }
+    return INT4MM_OK;
+}
+
+int64_t tuning(int key) { return (key >= 0 && key < TUNE_COUNT) ? g_tuning[key].load() : 0; }
+
+static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// Superset of the reference's host asserts (matmul_kernel.cu:379-416,435-439;
+// matvec_kernel.cu:307-337,356-360): every one of them is a returned error here.
+int validate_product(int bits, const void* outs, const void* matrix, const void* multiplier,
+                     const void* scales, const void* zeros, const void* sparse_mask,
+                     const int4mm_shape* sh, bool matvec) {
+    if (bits != 4 && bits != 3 && bits != 2) return INT4MM_ERR_BITS;
+    if (sh == nullptr) return INT4MM_ERR_NULL;
+    if (sparse_mask != nullptr && bits != 4) return INT4MM_ERR_SPARSE_BITS;
+    const int64_t B = sh->batch, M = sh->seq_len, K = sh->in_size, S = sh->out_size;
+    const int64_t R = sh->matrix_rows, G = sh->n_groups, g = sh->group_size;
+    if (B < 0 || M < 0 || K <= 0 || S <= 0 || R <= 0 || G <= 0) return INT4MM_ERR_SHAPE;
+    if (matvec && M != 1 && B * M * S != 0) return INT4MM_ERR_SHAPE;        // matvec_kernel.cu:323
+    if (K % 64 != 0 || S % 64 != 0) return INT4MM_ERR_SHAPE;                 // README.md:9
+    if (sparse_mask != nullptr) {
+        if (R * 16 != K) return INT4MM_ERR_SHAPE;                            // R*32*2/bits == K
+    } else {
+        if (R * 32 != K * bits) return INT4MM_ERR_SHAPE;
+    }
+    if (g == 0 || (g > 0 && g % 64 != 0)) return INT4MM_ERR_GROUP;           // matmul_kernel.cu:383
+    const int64_t geff = g < 0 ? ONE_GROUP : g;
+    if (G > (int64_t)1 << 40 || geff * G < K) return INT4MM_ERR_SHAPE;       // :413-414
+    if (K > ((int64_t)1 << 31) - 64 || S > ((int64_t)1 << 31) - 256 || M > ((int64_t)1 << 31) - 256 ||
+        B > 65535)
+        return INT4MM_ERR_SHAPE;
+    if (B * M * S == 0) return INT4MM_OK;
+    if (!outs || !matrix || !multiplier || !scales || !zeros) return INT4MM_ERR_NULL;
+    if (!aligned16(outs) || !aligned16(matrix) || !aligned16(multiplier) || !aligned16(scales) ||
+        !aligned16(zeros) || !aligned16(sparse_mask))
+        return INT4MM_ERR_ALIGN;
+    return INT4MM_OK;
+}
+
+__global__ void fill_zero_kernel(uint32_t* p, size_t n) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0u;
+}
+
+}  // namespace i4
+
+using namespace i4;
+
+extern "C" {
+
+const char* int4mm_error_string(int code) {
+    switch (code) {
+        case INT4MM_OK: return "ok";
+        case INT4MM_ERR_BITS: return "unsupported bit width (must be 4, 3 or 2)";
+        case INT4MM_ERR_SPARSE_BITS: return "16:32 sparsity is supported for int4 only";
+        case INT4MM_ERR_SHAPE: return "tensor shapes are inconsistent or not multiples of 64";
+        case INT4MM_ERR_GROUP: return "group_size must be negative or a positive multiple of 64";
+        case INT4MM_ERR_NULL: return "a required pointer is null";
+        case INT4MM_ERR_WORKSPACE: return "workspace missing or too small";
+        case INT4MM_ERR_LAUNCH: return "HIP launch failed";
+        case INT4MM_ERR_ALIGN: return "a device pointer is not 16-byte aligned";
+        default: return "unknown int4mm error";
+    }
+}
+
+int int4mm_last_hip_error(void) { return g_last_hip_error; }
+int int4mm_abi_version(void) { return 1; }
+
+// Benchmark/tuning hook: overrides a launch heuristic (0 restores the default).
+// Keys: 0 = matvec waves per workgroup, 1 = matvec 64-row units per wave,
+// 2 = reserved, 3 = matmul kernel variant.
+int int4mm_tune(int key, int64_t value) {
+    if (key < 0 || key >= TUNE_COUNT) return INT4MM_ERR_SHAPE;
+    g_tuning[key].store(value);
+    return INT4MM_OK;
+}
+
+// counters: one int32 per 64-column strip (+ slack); partial sums: up to 32
+// K-splits of fp32 [out_size]
+size_t int4mm_workspace_bytes(int64_t max_out_size) {
+    if (max_out_size < 0) max_out_size = 0;
+    size_t s = (size_t)((max_out_size + 255) / 256 * 256);
+    return 4096 + s * 4 * 32;
+}
+
+int int4mm_workspace_init(void* workspace, size_t workspace_bytes, void* stream) {
+    if (workspace == nullptr) return INT4MM_ERR_NULL;
+    if (workspace_bytes < 4096) return INT4MM_ERR_WORKSPACE;
+    size_t n = workspace_bytes / 4;
+    hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
+                       (hipStream_t)stream, (uint32_t*)workspace, n);
+    return check_launch("workspace_init");
+}
+
+}  // extern "C"

@@ -1,0 +1,94 @@
+// Shared device helpers for the gfx950 kernels: fp16 vector types, wave-level
+// reductions, the bit-exact dequantisation of one code, and host-side launch
+// bookkeeping.  Written for 64-lane wavefronts only.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/int4mm.h"
+
+namespace i4 {
+
+typedef _Float16 h16;
+typedef _Float16 h16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 h16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 h16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int WAVE = 64;
+constexpr int64_t ONE_GROUP = 0x0FFFFFFF;   // group_size < 0: a single group
+
+template <typename To, typename From>
+__device__ __forceinline__ To bitcast(From v) { return __builtin_bit_cast(To, v); }
+
+__device__ __forceinline__ h16x2 as_h2(uint32_t v) { return bitcast<h16x2>(v); }
+__device__ __forceinline__ uint32_t as_u32(h16x2 v) { return bitcast<uint32_t>(v); }
+__device__ __forceinline__ float lo_f32(uint32_t v) { return (float)as_h2(v).x; }
+__device__ __forceinline__ float hi_f32(uint32_t v) { return (float)as_h2(v).y; }
+
+// acc + a.x*b.x + a.y*b.y with an fp32 accumulator (v_dot2_f32_f16)
+__device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float acc) {
+    return __builtin_amdgcn_fdot2(as_h2(a), as_h2(b), acc, false);
+}
+
+// ---- wave-wide sum through DPP: quad swaps, half-row and row mirrors, then the
+// four row totals are combined from lanes 0/16/32/48.  Every lane gets the total.
+template <int CTRL>
+__device__ __forceinline__ float dpp_f32(float v) {
+    return bitcast<float>(__builtin_amdgcn_update_dpp(0, bitcast<int>(v), CTRL, 0xF, 0xF, true));
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+    v += dpp_f32<0xB1>(v);    // quad_perm [1,0,3,2]
+    v += dpp_f32<0x4E>(v);    // quad_perm [2,3,0,1]
+    v += dpp_f32<0x141>(v);   // row_half_mirror
+    v += dpp_f32<0x140>(v);   // row_mirror
+    int b = bitcast<int>(v);
+    float r0 = bitcast<float>(__builtin_amdgcn_readlane(b, 0));
+    float r1 = bitcast<float>(__builtin_amdgcn_readlane(b, 16));
+    float r2 = bitcast<float>(__builtin_amdgcn_readlane(b, 32));
+    float r3 = bitcast<float>(__builtin_amdgcn_readlane(b, 48));
+    return (r0 + r1) + (r2 + r3);
+}
+
+// ---- one code -> fp16 weight, the two roundings of the linear mode and the
+// single-rounded fused multiply-add of the exponent mode.
+template <int BITS>
+__device__ __forceinline__ h16 dequant_code(uint32_t q, h16 scale, h16 zero) {
+    if (scale >= (h16)0.0f) {
+        h16 d = (h16)(float)q - zero;       // fp16 subtract, one rounding
+        return d * scale;                    // fp16 multiply, one rounding
+    }
+    constexpr uint32_t EXP_MSK = (1u << (BITS - 1)) - 1u, SGN = 1u << (BITS - 1);
+    int iv = 1 << (q & EXP_MSK);
+    if (q & SGN) iv = -iv;
+    return __builtin_fmaf16((h16)(float)iv, -scale, zero);
+}
+
+// value a code stands for before scale/zero are applied: q in linear mode,
+// +-2^(low bits) in exponent mode
+template <int BITS>
+__device__ __forceinline__ float code_value(uint32_t q, bool exponent_mode) {
+    constexpr uint32_t EXP_MSK = (1u << (BITS - 1)) - 1u, SGN = 1u << (BITS - 1);
+    float lin = (float)q;
+    float ex = (float)(1u << (q & EXP_MSK));
+    ex = (q & SGN) ? -ex : ex;
+    return exponent_mode ? ex : lin;
+}
+
+// ---- host side
+struct LaunchStatus { int code; hipError_t hip; };
+
+int check_launch(const char* what);           // returns INT4MM_OK or INT4MM_ERR_LAUNCH
+int validate_product(int bits, const void* outs, const void* matrix, const void* multiplier,
+                     const void* scales, const void* zeros, const void* sparse_mask,
+                     const int4mm_shape* sh, bool matvec);
+int64_t tuning(int key);                       // see int4mm_tune
+enum TuneKey { TUNE_MV_WAVES = 0, TUNE_MV_UNITS = 1, TUNE_MV_SPLITS = 2, TUNE_MM_VARIANT = 3,
+               TUNE_COUNT = 8 };
+
+}  // namespace i4

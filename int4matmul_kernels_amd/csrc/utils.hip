@@ -1,0 +1,233 @@
+// Pack / unpack / dequantise helpers for the packed weight formats.  These are
+// integer kernels bound by HBM traffic: one thread owns one (32-row block,
+// column) cell, lanes run along the column index so every global access of the
+// [rows, S] matrices is coalesced.
+#include "common.h"
+
+namespace i4 {
+
+// 32 codes of one column, blocks of 32 rows: the shared decode step.
+template <int BITS, bool SPARSE>
+__device__ __forceinline__ void decode_block32(const uint32_t* __restrict__ matrix,
+                                               const uint32_t* __restrict__ mask, int64_t S,
+                                               int64_t blk, int64_t s, uint32_t codes[32],
+                                               uint32_t& keep) {
+    keep = 0xFFFFFFFFu;
+    if constexpr (SPARSE) {
+        const uint32_t lo = matrix[(2 * blk) * S + s], hi = matrix[(2 * blk + 1) * S + s];
+        uint64_t v = (uint64_t)lo | ((uint64_t)hi << 32);
+        keep = mask[blk * S + s];
+#pragma unroll
+        for (int t = 0; t < 32; ++t) {
+            const bool k = (keep >> t) & 1u;
+            codes[t] = k ? (uint32_t)(v & 0xF) : 0u;
+            v >>= k ? 4 : 0;
+        }
+    } else if constexpr (BITS == 3) {
+        const uint32_t w0 = matrix[(3 * blk) * S + s], w1 = matrix[(3 * blk + 1) * S + s],
+                       w2 = matrix[(3 * blk + 2) * S + s];
+        const uint64_t lo = (uint64_t)w0 | ((uint64_t)w1 << 32);   // stream bits 0..63
+        const uint64_t hi = (uint64_t)w1 | ((uint64_t)w2 << 32);   // stream bits 32..95
+#pragma unroll
+        for (int t = 0; t < 32; ++t) {
+            const int pos = 3 * t;
+            codes[t] = pos + 3 <= 64 ? (uint32_t)(lo >> pos) & 7u : (uint32_t)(hi >> (pos - 32)) & 7u;
+        }
+    } else {
+        constexpr int PER = 32 / BITS;
+#pragma unroll
+        for (int i = 0; i < BITS; ++i) {
+            uint32_t v = matrix[(BITS * blk + i) * S + s];
+#pragma unroll
+            for (int j = 0; j < PER; ++j) {
+                codes[i * PER + j] = v & ((1u << BITS) - 1u);
+                v >>= BITS;
+            }
+        }
+    }
+}
+
+template <int BITS, bool SPARSE>
+__global__ __launch_bounds__(256) void unpack_kernel(uint8_t* __restrict__ codes_out,
+                                                     uint8_t* __restrict__ keep_out,
+                                                     const uint32_t* __restrict__ matrix,
+                                                     const uint32_t* __restrict__ mask, int64_t K,
+                                                     int64_t S) {
+    const int64_t s = (int64_t)blockIdx.x * blockDim.x + threadIdx.x, blk = blockIdx.y;
+    if (s >= S) return;
+    uint32_t codes[32], keep;
+    decode_block32<BITS, SPARSE>(matrix, mask, S, blk, s, codes, keep);
+#pragma unroll
+    for (int t = 0; t < 32; ++t) {
+        codes_out[(blk * 32 + t) * S + s] = (uint8_t)codes[t];
+        if (keep_out) keep_out[(blk * 32 + t) * S + s] = (uint8_t)((keep >> t) & 1u);
+    }
+}
+
+template <int BITS, bool SPARSE>
+__global__ __launch_bounds__(256) void dequantize_kernel(h16* __restrict__ w_out,
+                                                         const uint32_t* __restrict__ matrix,
+                                                         const uint32_t* __restrict__ mask,
+                                                         const h16* __restrict__ scales,
+                                                         const h16* __restrict__ zeros, int64_t K,
+                                                         int64_t S, int64_t group_size) {
+    const int64_t s = (int64_t)blockIdx.x * blockDim.x + threadIdx.x, blk = blockIdx.y;
+    if (s >= S) return;
+    uint32_t codes[32], keep;
+    decode_block32<BITS, SPARSE>(matrix, mask, S, blk, s, codes, keep);
+    const int64_t gi = (blk * 32) / group_size;      // group_size is a multiple of 64
+    const h16 sc = scales[gi * S + s], ze = zeros[gi * S + s];
+#pragma unroll
+    for (int t = 0; t < 32; ++t) {
+        h16 w = dequant_code<BITS>(codes[t], sc, ze);
+        if (SPARSE && !((keep >> t) & 1u)) w = (h16)0.0f;
+        w_out[(blk * 32 + t) * S + s] = w;
+    }
+}
+
+// codes uint8 [K, S] -> packed words, LSB-first bitstream of 32 codes per block
+template <int BITS>
+__global__ __launch_bounds__(256) void dense_pack_kernel(uint32_t* __restrict__ matrix_out,
+                                                         const uint8_t* __restrict__ codes_in,
+                                                         int64_t K, int64_t S) {
+    const int64_t s = (int64_t)blockIdx.x * blockDim.x + threadIdx.x, blk = blockIdx.y;
+    if (s >= S) return;
+    uint64_t lo = 0, hi = 0;                          // stream bits 0..63 and 64..127
+#pragma unroll
+    for (int t = 0; t < 32; ++t) {
+        const uint64_t c = codes_in[(blk * 32 + t) * S + s] & ((1u << BITS) - 1u);
+        const int pos = BITS * t;
+        if (pos < 64) {
+            lo |= c << pos;
+            if (pos + BITS > 64) hi |= c >> (64 - pos);
+        } else {
+            hi |= c << (pos - 64);
+        }
+    }
+    const uint32_t w[4] = {(uint32_t)lo, (uint32_t)(lo >> 32), (uint32_t)hi, (uint32_t)(hi >> 32)};
+#pragma unroll
+    for (int i = 0; i < BITS; ++i) matrix_out[(BITS * blk + i) * S + s] = w[i];
+}
+
+// 16:32 packer.  Inputs are in the [S, K] orientation (row = output column), so
+// each thread reads the 32 consecutive bytes of its cell and writes three words
+// with lanes along the column index.
+__global__ __launch_bounds__(256) void sparse_pack_kernel(uint32_t* __restrict__ wt_outs,
+                                                          uint32_t* __restrict__ msk_outs,
+                                                          const uint8_t* __restrict__ wt_in,
+                                                          const uint8_t* __restrict__ msk_in,
+                                                          int64_t S, int64_t K,
+                                                          int* __restrict__ bad_blocks) {
+    const int64_t s = (int64_t)blockIdx.x * blockDim.x + threadIdx.x, blk = blockIdx.y;
+    if (s >= S) return;
+    const u32x4* wp = reinterpret_cast<const u32x4*>(wt_in + s * K + blk * 32);
+    const u32x4* mp = reinterpret_cast<const u32x4*>(msk_in + s * K + blk * 32);
+    const u32x4 wa = wp[0], wb = wp[1], ma = mp[0], mb = mp[1];
+    const uint32_t wv[8] = {wa.x, wa.y, wa.z, wa.w, wb.x, wb.y, wb.z, wb.w};
+    const uint32_t mv[8] = {ma.x, ma.y, ma.z, ma.w, mb.x, mb.y, mb.z, mb.w};
+    uint32_t bmsk = 0;
+    uint64_t v = 0;
+    int rank = 0;
+#pragma unroll
+    for (int t = 0; t < 32; ++t) {
+        const uint32_t code = (wv[t >> 2] >> (8 * (t & 3))) & 0xFu;
+        const bool k = ((mv[t >> 2] >> (8 * (t & 3))) & 0xFFu) > 0;
+        if (k) {
+            bmsk |= 1u << t;
+            if (rank < 16) v |= (uint64_t)code << (4 * rank);
+            ++rank;
+        }
+    }
+    msk_outs[blk * S + s] = bmsk;
+    wt_outs[(2 * blk) * S + s] = (uint32_t)v;
+    wt_outs[(2 * blk + 1) * S + s] = (uint32_t)(v >> 32);
+    if (rank != 16 && bad_blocks) atomicAdd(bad_blocks, 1);
+}
+
+static dim3 cell_grid(int64_t S, int64_t K) { return dim3((unsigned)((S + 255) / 256), (unsigned)(K / 32)); }
+
+}  // namespace i4
+
+using namespace i4;
+
+extern "C" {
+
+int int4mm_sparse_pack(void* wt_outs, void* msk_outs, const void* wt_in, const void* msk_in,
+                       int64_t out_size, int64_t in_size, void* bad_blocks, void* stream) {
+    if (out_size < 0 || in_size < 0 || in_size % 32 != 0) return INT4MM_ERR_SHAPE;
+    if (in_size / 32 > 65535) return INT4MM_ERR_SHAPE;
+    if (out_size == 0 || in_size == 0) return INT4MM_OK;
+    if (!wt_outs || !msk_outs || !wt_in || !msk_in) return INT4MM_ERR_NULL;
+    if (((uintptr_t)wt_in | (uintptr_t)msk_in) & 15u) return INT4MM_ERR_ALIGN;
+    hipLaunchKernelGGL(sparse_pack_kernel, cell_grid(out_size, in_size), dim3(256), 0,
+                       (hipStream_t)stream, (uint32_t*)wt_outs, (uint32_t*)msk_outs,
+                       (const uint8_t*)wt_in, (const uint8_t*)msk_in, out_size, in_size,
+                       (int*)bad_blocks);
+    return check_launch("sparse_pack");
+}
+
+int int4mm_dense_pack(int bits, void* matrix_out, const void* codes_in, int64_t in_size,
+                      int64_t out_size, void* stream) {
+    if (bits != 4 && bits != 3 && bits != 2) return INT4MM_ERR_BITS;
+    if (out_size < 0 || in_size < 0 || in_size % 32 != 0 || in_size / 32 > 65535)
+        return INT4MM_ERR_SHAPE;
+    if (out_size == 0 || in_size == 0) return INT4MM_OK;
+    if (!matrix_out || !codes_in) return INT4MM_ERR_NULL;
+    const dim3 grid = cell_grid(out_size, in_size), block(256);
+    hipStream_t st = (hipStream_t)stream;
+    uint32_t* o = (uint32_t*)matrix_out;
+    const uint8_t* c = (const uint8_t*)codes_in;
+    if (bits == 4) hipLaunchKernelGGL(dense_pack_kernel<4>, grid, block, 0, st, o, c, in_size, out_size);
+    if (bits == 3) hipLaunchKernelGGL(dense_pack_kernel<3>, grid, block, 0, st, o, c, in_size, out_size);
+    if (bits == 2) hipLaunchKernelGGL(dense_pack_kernel<2>, grid, block, 0, st, o, c, in_size, out_size);
+    return check_launch("dense_pack");
+}
+
+int int4mm_unpack(int bits, void* codes_out, void* keep_out, const void* matrix,
+                  const void* sparse_mask, int64_t in_size, int64_t out_size, void* stream) {
+    if (bits != 4 && bits != 3 && bits != 2) return INT4MM_ERR_BITS;
+    if (sparse_mask && bits != 4) return INT4MM_ERR_SPARSE_BITS;
+    if (out_size < 0 || in_size < 0 || in_size % 32 != 0 || in_size / 32 > 65535)
+        return INT4MM_ERR_SHAPE;
+    if (out_size == 0 || in_size == 0) return INT4MM_OK;
+    if (!codes_out || !matrix) return INT4MM_ERR_NULL;
+    const dim3 grid = cell_grid(out_size, in_size), block(256);
+    hipStream_t st = (hipStream_t)stream;
+    uint8_t* o = (uint8_t*)codes_out;
+    uint8_t* k = (uint8_t*)keep_out;
+    const uint32_t* m = (const uint32_t*)matrix;
+    const uint32_t* msk = (const uint32_t*)sparse_mask;
+    if (msk) hipLaunchKernelGGL((unpack_kernel<4, true>), grid, block, 0, st, o, k, m, msk, in_size, out_size);
+    else if (bits == 4) hipLaunchKernelGGL((unpack_kernel<4, false>), grid, block, 0, st, o, k, m, msk, in_size, out_size);
+    else if (bits == 3) hipLaunchKernelGGL((unpack_kernel<3, false>), grid, block, 0, st, o, k, m, msk, in_size, out_size);
+    else hipLaunchKernelGGL((unpack_kernel<2, false>), grid, block, 0, st, o, k, m, msk, in_size, out_size);
+    return check_launch("unpack");
+}
+
+int int4mm_dequantize(int bits, void* w_out, const void* matrix, const void* scales,
+                      const void* zeros, const void* sparse_mask, int64_t in_size,
+                      int64_t out_size, int64_t n_groups, int64_t group_size, void* stream) {
+    if (bits != 4 && bits != 3 && bits != 2) return INT4MM_ERR_BITS;
+    if (sparse_mask && bits != 4) return INT4MM_ERR_SPARSE_BITS;
+    if (out_size < 0 || in_size < 0 || in_size % 64 != 0 || in_size / 32 > 65535 || n_groups <= 0)
+        return INT4MM_ERR_SHAPE;
+    if (group_size == 0 || (group_size > 0 && group_size % 64 != 0)) return INT4MM_ERR_GROUP;
+    const int64_t g = group_size < 0 ? ONE_GROUP : group_size;
+    if (n_groups > ((int64_t)1 << 40) || g * n_groups < in_size) return INT4MM_ERR_SHAPE;
+    if (out_size == 0 || in_size == 0) return INT4MM_OK;
+    if (!w_out || !matrix || !scales || !zeros) return INT4MM_ERR_NULL;
+    const dim3 grid = cell_grid(out_size, in_size), block(256);
+    hipStream_t st = (hipStream_t)stream;
+    h16* o = (h16*)w_out;
+    const uint32_t* m = (const uint32_t*)matrix;
+    const uint32_t* msk = (const uint32_t*)sparse_mask;
+    const h16* sc = (const h16*)scales;
+    const h16* ze = (const h16*)zeros;
+    if (msk) hipLaunchKernelGGL((dequantize_kernel<4, true>), grid, block, 0, st, o, m, msk, sc, ze, in_size, out_size, g);
+    else if (bits == 4) hipLaunchKernelGGL((dequantize_kernel<4, false>), grid, block, 0, st, o, m, msk, sc, ze, in_size, out_size, g);
+    else if (bits == 3) hipLaunchKernelGGL((dequantize_kernel<3, false>), grid, block, 0, st, o, m, msk, sc, ze, in_size, out_size, g);
+    else hipLaunchKernelGGL((dequantize_kernel<2, false>), grid, block, 0, st, o, m, msk, sc, ze, in_size, out_size, g);
+    return check_launch("dequantize");
+}
+
+}  // extern "C"

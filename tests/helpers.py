@@ -1,0 +1,95 @@
+"""Shared helpers for the GPU parity tests: move an oracle problem to the GPU
+and call the HIP path either through the C ABI (ctypes) or through the
+``int4matmul`` extension module."""
+import numpy as np
+import torch
+
+import int4matmul_kernels_amd as pkg
+from int4matmul_kernels_amd import capi
+from oracle import oracle as O
+
+DEV = "cuda"
+
+
+def t(a, dev=DEV):
+    if a is None:
+        return None
+    return torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+
+
+def dev_problem(p):
+    return dict(matrix=t(p["matrix"]), mask=t(p["sparse_mask"]), states=t(p["states"]),
+                scales=t(p["scales"]), zeros=t(p["zeros"]))
+
+
+def run_capi(p, d, kind, outs_init=None):
+    B, M, S = p["B"], p["M"], p["S"]
+    outs = torch.zeros((B, M, S), dtype=torch.float16, device=DEV) if outs_init is None \
+        else t(outs_init).clone()
+    ws = capi.new_workspace(S)
+    fn = capi.matvec if kind == "vec" else capi.matmul
+    fn(p["bits"], outs, d["matrix"], d["states"], d["scales"], d["zeros"], p["group_size"],
+       d["mask"], ws)
+    torch.cuda.synchronize()
+    return outs.cpu().numpy()
+
+
+def run_ext(p, d, outs_init=None, fn_name="quant_matmul"):
+    ext = pkg.load_extension()
+    B, M, S = p["B"], p["M"], p["S"]
+    outs = torch.zeros((B, M, S), dtype=torch.float16, device=DEV) if outs_init is None \
+        else t(outs_init).clone()
+    args = (outs, d["matrix"], d["states"], d["scales"], d["zeros"], p["group_size"], d["mask"])
+    if fn_name == "quant_matmul":
+        ext.quant_matmul(p["bits"], *args)
+    else:
+        getattr(ext, fn_name)(*args)
+    torch.cuda.synchronize()
+    return outs.cpu().numpy()
+
+
+def oracles(p):
+    """(exact fp64 product on the fp16 weights, fp32 dequantise-then-matmul)"""
+    w16 = O.dequantize_matrix(p["bits"], p["matrix"], p["scales"], p["zeros"], p["group_size"],
+                              p["sparse_mask"])
+    x = p["states"].reshape(-1, p["K"])
+    exact = O.matmul_exact(x, w16).reshape(p["B"], p["M"], p["S"])
+    linear_only = bool(np.all(p["scales"] >= 0))
+    if linear_only:
+        w32 = O.dequantize_matrix_fp32(p["bits"], p["matrix"], p["scales"], p["zeros"],
+                                       p["group_size"], p["sparse_mask"])
+        f32 = O.matmul_fp32(x, w32).reshape(p["B"], p["M"], p["S"])
+    else:
+        f32 = exact.astype(np.float32)
+    return exact, f32
+
+
+# Tolerances (stated once, used by every product test):
+#  * against fp32 dequantise-then-matmul: max relative error 1e-2, the bar of the
+#    build's north star, denominators floored at the RMS of the true outputs;
+#  * against the exact (float64) product on the fp16 weights the reference
+#    multiplies: 2e-3 for the matmul, whose weights are those fp16 values bit for
+#    bit (what is left is fp32 summation order and the fp16 output rounding,
+#    4.9e-4 relative); 6e-3 for the matvec, which applies scale and zero in fp32
+#    per group instead of rounding every weight to fp16 twice, so it differs
+#    from that product by the weights' own rounding noise (and is closer to the
+#    fp32 oracle than the reference is);
+#  * the reference's own gate: mean relative error <= 0.1 (kernel_test.py:344-348).
+TOL_F32 = 1e-2
+TOL_EXACT = 6e-3          # matvec
+TOL_EXACT_MTX = 2e-3      # matmul
+TOL_MEAN = 0.1
+
+
+def assert_product_close(got, exact, f32, prior=None, kind="vec"):
+    if prior is not None:
+        exact = exact + prior.astype(np.float64)
+        f32 = f32 + prior.astype(np.float32)
+    assert np.all(np.isfinite(got.astype(np.float32)))
+    e1 = O.max_rel_error(exact, got)
+    e2 = O.max_rel_error(f32, got)
+    e3 = O.mean_rel_error(f32, got)
+    assert e1 < (TOL_EXACT if kind == "vec" else TOL_EXACT_MTX), f"vs exact product: {e1}"
+    assert e2 < TOL_F32, f"vs fp32 oracle: {e2}"
+    assert e3 < TOL_MEAN, f"mean relative error: {e3}"
+    return e1, e2, e3
