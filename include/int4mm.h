@@ -67,7 +67,8 @@ INT4MM_API int int4mm_abi_version(void);
 
 /* Benchmark / tuning hook, not part of the drop-in boundary: overrides a launch
  * heuristic process-wide (value 0 restores the default).  key 0 = matvec waves
- * per workgroup, 1 = matvec 64-row units per wave, 3 = matmul kernel variant. */
+ * per workgroup, 1 = matvec 64-row units per lane group, 2 = matvec lane groups per
+ * wave (1, 2, 4), 3 = matmul kernel variant, 4 = matvec: 1 disables prefetch. */
 INT4MM_API int int4mm_tune(int key, int64_t value);
 
 /* Shape of one product.  matrix_rows = R, n_groups = G (rows of scales/zeros).

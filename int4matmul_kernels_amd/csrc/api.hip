@@ -84,20 +84,20 @@ int int4mm_last_hip_error(void) { return g_last_hip_error; }
 int int4mm_abi_version(void) { return 1; }
 
 // Benchmark/tuning hook: overrides a launch heuristic (0 restores the default).
-// Keys: 0 = matvec waves per workgroup, 1 = matvec 64-row units per wave,
-// 2 = reserved, 3 = matmul kernel variant.
+// Keys: 0 = matvec waves per workgroup, 1 = matvec units per lane group,
+// 2 = matvec lane groups per wave (1, 2 or 4), 3 = matmul kernel variant,
+// 4 = matvec: 1 disables the software prefetch.
 int int4mm_tune(int key, int64_t value) {
     if (key < 0 || key >= TUNE_COUNT) return INT4MM_ERR_SHAPE;
     g_tuning[key].store(value);
     return INT4MM_OK;
 }
 
-// counters: one int32 per 64-column strip (+ slack); partial sums: up to 32
-// K-splits of fp32 [out_size]
+// hand-over slots of the matvec: up to 32 K-splits x out_size x {fp32, flag}
 size_t int4mm_workspace_bytes(int64_t max_out_size) {
     if (max_out_size < 0) max_out_size = 0;
     size_t s = (size_t)((max_out_size + 255) / 256 * 256);
-    return 4096 + s * 4 * 32;
+    return 4096 + s * 8 * 32;
 }
 
 int int4mm_workspace_init(void* workspace, size_t workspace_bytes, void* stream) {

@@ -88,7 +88,7 @@ int validate_product(int bits, const void* outs, const void* matrix, const void*
                      const void* scales, const void* zeros, const void* sparse_mask,
                      const int4mm_shape* sh, bool matvec);
 int64_t tuning(int key);                       // see int4mm_tune
-enum TuneKey { TUNE_MV_WAVES = 0, TUNE_MV_UNITS = 1, TUNE_MV_SPLITS = 2, TUNE_MM_VARIANT = 3,
+enum TuneKey { TUNE_MV_WAVES = 0, TUNE_MV_UNITS = 1, TUNE_MV_LK = 2, TUNE_MM_VARIANT = 3, TUNE_MV_NOPF = 4,
                TUNE_COUNT = 8 };
 
 }  // namespace i4

@@ -2,31 +2,40 @@
 //
 // Bandwidth-bound streaming kernel.  The packed matrix is [rows, S] with the
 // column index contiguous, so lanes own columns: a lane reads 16 bytes = the
-// packed words of 4 adjacent columns of one packed row, a wavefront reads
-// 1 KiB contiguous per row.  K is cut into 64-row "units" (the granularity of
-// quantisation groups); a wave walks a run of units, a workgroup's waves walk
-// adjacent runs, grid.y cuts K further.  Partial sums meet in LDS, and across
-// workgroups through fp32 slots in the workspace with an arrival counter: the
-// last workgroup of a column strip adds the slots in a fixed order, adds the
-// prior contents of outs and writes fp16 -- one kernel, deterministic.
+// packed words of 4 adjacent columns of one packed row.  K is cut into 64-row
+// "units" (the granularity of quantisation groups).  A wavefront is LK lane
+// groups of 64/LK lanes; each lane group streams its own units, so one load
+// instruction fetches LK contiguous segments of (64/LK)*16 bytes.  A workgroup
+// owns a strip of (64/LK)*4 columns and a range of units; grid.y cuts K further.
 //
-// Arithmetic: the states x are wave-uniform, so they travel through scalar
-// registers.  For int4/int2 the codes are never converted one by one: a mask
-// and an OR turn two fields of a word into a half2 whose lanes are 2^e + q
-// ("magic" exponents chosen so that the field lands on the units of the
-// mantissa), v_dot2_f32_f16 multiplies that pair by the matching pair of states
-// into an fp32 accumulator, and the constant part sum_k 2^e_k * x_k is removed
-// once per unit.  Per (group, column):  y += s * (sum_k x_k q_k - z * sum_k x_k),
-// which is the exact value of sum_k x_k (q_k - z) s; the fp16 roundings that the
-// reference applies to each weight are not reproduced here (they are in the
-// dequantise helper, which is bit-exact).
+// The states x of the workgroup's K range are staged once in LDS, already
+// permuted into the half2 pairs the decode produces, together with per-unit
+// sums; every lane of a lane group reads the same LDS address (a broadcast).
+//
+// Arithmetic (int4 / int2): codes are never converted one by one.  A mask and
+// an OR turn two fields of a word into a half2 whose lanes are 2^e + q ("magic"
+// exponents chosen so that the field lands on the units of the mantissa),
+// v_dot2_f32_f16 multiplies the pair by the matching pair of states into an fp32
+// accumulator, and the constant part sum_k 2^e_k x_k is removed once per unit.
+// Per (unit, column):  y += s * (sum_k x_k q_k - z * sum_k x_k), the exact value
+// of sum_k x_k (q_k - z) s; the two fp16 roundings the reference applies to each
+// weight are not reproduced here (the dequantise helper is the bit-exact one).
+// Columns whose scale is negative (exponent quantisation) are left out of the
+// fast loop and handled by a second, general loop that only runs if any exist.
+//
+// Partial sums meet in LDS; across workgroups they meet in 8-byte slots of the
+// workspace {fp32 partial, flag}: a workgroup publishes its slots with
+// device-scope write-through stores and leaves; the workgroup with the highest
+// index of the strip polls the slots, adds them in a fixed order
+// (deterministic), adds the prior contents of outs, writes fp16 and clears the
+// slots.  No cache-wide fence and no read-modify-write atomics are used.
 #include "common.h"
 
 namespace i4 {
 
-constexpr int MV_MAX_WAVES = 16;
-constexpr int MV_COLS = 256;          // columns per wave: 64 lanes x 4
-constexpr int MV_MAX_SPLITS = 32;
+constexpr int MV_MAX_WAVES = 8;
+constexpr int MV_MAX_SPLITS = 32;          // slots per column in the workspace
+constexpr int MV_MAX_UNITS_WG = 1024;     // LDS staging: 128 B of states + 8 B of sums per unit
 
 struct MatvecArgs {
     h16* outs;
@@ -35,298 +44,471 @@ struct MatvecArgs {
     const h16* x;
     const h16* scales;
     const h16* zeros;
-    float* partials;        // [splits][S]
-    int* counters;          // [strips]
+    uint64_t* slots;        // [splits - 1][S] hand-over slots {partial sum, flag}
     int K, S;
     int units_total;        // K / 64
-    int units_per_wave;
+    int units_per_wg;
     int group_units;        // group size in units (>= 1); huge for a single group
     int splits;             // == gridDim.y
 };
 
-typedef const uint32_t __attribute__((address_space(4))) * const_u32p;
-
-__device__ __forceinline__ const_u32p to_const(const void* p) {
-    return (const_u32p)(uintptr_t)p;
-}
-
 // ------------------------------------------------------------------ formats
-// Packed rows per 64-row unit, and how one unit is held in registers.
 template <int BITS, bool SPARSE> struct Fmt;
-template <> struct Fmt<4, false> { static constexpr int ROWS = 8, MROWS = 0; };
-template <> struct Fmt<3, false> { static constexpr int ROWS = 6, MROWS = 0; };
-template <> struct Fmt<2, false> { static constexpr int ROWS = 4, MROWS = 0; };
-template <> struct Fmt<4, true>  { static constexpr int ROWS = 4, MROWS = 2; };
+template <> struct Fmt<4, false> { static constexpr int ROWS = 8, MROWS = 0; static constexpr bool FAST = true; };
+template <> struct Fmt<3, false> { static constexpr int ROWS = 6, MROWS = 0; static constexpr bool FAST = false; };
+template <> struct Fmt<2, false> { static constexpr int ROWS = 4, MROWS = 0; static constexpr bool FAST = true; };
+template <> struct Fmt<4, true>  { static constexpr int ROWS = 4, MROWS = 2; static constexpr bool FAST = false; };
 
 template <int BITS, bool SPARSE>
 struct Unit {
     u32x4 w[Fmt<BITS, SPARSE>::ROWS];
     u32x4 m[Fmt<BITS, SPARSE>::MROWS == 0 ? 1 : Fmt<BITS, SPARSE>::MROWS];
     u32x2 sc, ze;            // fp16 scales / zeros of the lane's 4 columns
-    float xl;                // x[k0 + lane] for the wave-wide sums
 };
 
 template <int BITS, bool SPARSE>
-__device__ __forceinline__ void load_unit(Unit<BITS, SPARSE>& u, const MatvecArgs& a, int unit,
-                                          int col, bool col_ok, int lane) {
+__device__ __forceinline__ void load_unit(Unit<BITS, SPARSE>& u, const MatvecArgs& a, int unit, int col) {
     constexpr int ROWS = Fmt<BITS, SPARSE>::ROWS, MROWS = Fmt<BITS, SPARSE>::MROWS;
     const int64_t S = a.S;
-    if (col_ok) {
-        const uint32_t* p = a.matrix + (int64_t)unit * ROWS * S + col;
+    const uint32_t* p = a.matrix + (int64_t)unit * ROWS * S + col;
 #pragma unroll
-        for (int r = 0; r < ROWS; ++r) u.w[r] = *reinterpret_cast<const u32x4*>(p + r * S);
-        if constexpr (MROWS > 0) {
-            const uint32_t* q = a.mask + (int64_t)unit * MROWS * S + col;
+    for (int r = 0; r < ROWS; ++r) u.w[r] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p + r * S));
+    if constexpr (MROWS > 0) {
+        const uint32_t* q = a.mask + (int64_t)unit * MROWS * S + col;
 #pragma unroll
-            for (int r = 0; r < MROWS; ++r) u.m[r] = *reinterpret_cast<const u32x4*>(q + r * S);
-        }
-        const int64_t gofs = (int64_t)(unit / a.group_units) * S + col;
-        u.sc = *reinterpret_cast<const u32x2*>(a.scales + gofs);
-        u.ze = *reinterpret_cast<const u32x2*>(a.zeros + gofs);
-    } else {
-#pragma unroll
-        for (int r = 0; r < ROWS; ++r) u.w[r] = u32x4{0, 0, 0, 0};
-        if constexpr (MROWS > 0) {
-#pragma unroll
-            for (int r = 0; r < MROWS; ++r) u.m[r] = u32x4{0, 0, 0, 0};
-        }
-        u.sc = u32x2{0, 0};
-        u.ze = u32x2{0, 0};
+        for (int r = 0; r < MROWS; ++r) u.m[r] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(q + r * S));
     }
-    u.xl = (float)a.x[unit * 64 + lane];
+    const int64_t gofs = (int64_t)(unit / a.group_units) * S + col;
+    u.sc = *reinterpret_cast<const u32x2*>(a.scales + gofs);
+    u.ze = *reinterpret_cast<const u32x2*>(a.zeros + gofs);
 }
 
-__device__ __forceinline__ uint32_t pack_lo(uint32_t a, uint32_t b) { return (a & 0xFFFFu) | (b << 16); }
-__device__ __forceinline__ uint32_t pack_hi(uint32_t a, uint32_t b) { return (a >> 16) | (b & 0xFFFF0000u); }
-
-// Slow, fully general accumulation of one unit (any format, either quantisation
-// mode).  acc[c] = sum over kept k of x_k * value(q_k); xs[c] = sum over kept k
-// of x_k.
-template <int BITS, bool SPARSE>
-__device__ __forceinline__ void unit_generic(const Unit<BITS, SPARSE>& u, const_u32p xw,
-                                             const bool expo[4], float acc[4], float xs[4]) {
-#pragma unroll
-    for (int c = 0; c < 4; ++c) { acc[c] = 0.f; xs[c] = 0.f; }
-#pragma unroll
-    for (int hb = 0; hb < 2; ++hb) {                 // two 32-row blocks
-#pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            uint32_t codes[32];
-            uint32_t keep = 0xFFFFFFFFu;
-            if constexpr (SPARSE) {
-                uint64_t v = (uint64_t)u.w[2 * hb][c] | ((uint64_t)u.w[2 * hb + 1][c] << 32);
-                keep = u.m[hb][c];
-#pragma unroll
-                for (int t = 0; t < 32; ++t) {
-                    const bool k = (keep >> t) & 1u;
-                    codes[t] = (uint32_t)v & 0xFu;
-                    v >>= k ? 4 : 0;
-                }
-            } else if constexpr (BITS == 3) {
-                const uint64_t lo = (uint64_t)u.w[3 * hb][c] | ((uint64_t)u.w[3 * hb + 1][c] << 32);
-                const uint64_t hi = (uint64_t)u.w[3 * hb + 1][c] | ((uint64_t)u.w[3 * hb + 2][c] << 32);
-#pragma unroll
-                for (int t = 0; t < 32; ++t) {
-                    const int pos = 3 * t;
-                    codes[t] = pos + 3 <= 64 ? (uint32_t)(lo >> pos) & 7u
-                                             : (uint32_t)(hi >> (pos - 32)) & 7u;
-                }
-            } else {
-                constexpr int PER = 32 / BITS;
-#pragma unroll
-                for (int i = 0; i < BITS; ++i) {
-                    uint32_t v = u.w[BITS * hb + i][c];
-#pragma unroll
-                    for (int j = 0; j < PER; ++j) { codes[i * PER + j] = v & ((1u << BITS) - 1u); v >>= BITS; }
-                }
-            }
-#pragma unroll
-            for (int t = 0; t < 32; ++t) {
-                const uint32_t xpair = xw[hb * 16 + t / 2];
-                const float xv = (t & 1) ? hi_f32(xpair) : lo_f32(xpair);
-                const float val = code_value<BITS>(codes[t], expo[c]);
-                const bool k = !SPARSE || ((keep >> t) & 1u);
-                acc[c] += k ? xv * val : 0.f;
-                if (SPARSE) xs[c] += k ? xv : 0.f;
-            }
-        }
-    }
+// (w & mask) | magic is one VALU op (v_and_or_b32) only when both constants sit
+// in registers: a VOP3 instruction of this ISA cannot carry two literals.  The
+// constants are therefore materialised once through an opaque move, and the
+// expression itself is left to the compiler (so that it also tracks the
+// VALU -> MFMA operand hazards, which it cannot do through inline assembly).
+__device__ __forceinline__ uint32_t in_vgpr(uint32_t literal) {
+    uint32_t r;
+    asm("v_mov_b32 %0, %1" : "=v"(r) : "s"(literal));
+    return r;
+}
+__device__ __forceinline__ uint32_t and_or(uint32_t w, uint32_t mask, uint32_t magic) {
+    return (w & mask) | magic;
 }
 
-// Fast int4 path.  Word bits: code j at 4j.  Pairs (j, j+4) sit at equal offsets
-// in the two halves of the word; offsets 0 and 4 are inside the fp16 mantissa, so
+// ---- fast paths.  xp points at the unit's staged states (LDS).
+//
+// The multiply-accumulate itself runs on the matrix core, which is otherwise
+// idle in a matvec and executes beside the VALU: v_mfma_f32_4x4x4_16B_f16 is 16
+// independent 4x4x4 products, block b = lanes 4b..4b+3; lane 4b+j supplies
+// column j of B (4 consecutive k) and lane 4b+i row i of A.  Every lane passes
+// the same four states as its A row and its own four weights as its B column,
+// so each of the lane's 4 result registers holds its column's dot product.
+typedef _Float16 h16x4v __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ f32x4 mma4(uint32_t a0, uint32_t a1, uint32_t b0, uint32_t b1, f32x4 c) {
+    const u32x2 a = {a0, a1}, b = {b0, b1};
+    return __builtin_amdgcn_mfma_f32_4x4x4f16(bitcast<h16x4v>(a), bitcast<h16x4v>(b), c, 0, 0, 0);
+}
+
+// int4: word bits: code j at 4j.  Pairs (j, j+4) sit at equal offsets in the two
+// halves of the word; offsets 0 and 4 are inside the fp16 mantissa, so
 //   (w & 0x000F000F) | 0x64006400 = {1024 + q0, 1024 + q4}
 //   (w & 0x00F000F0) | 0x54005400 = {  64 + q1,   64 + q5}
-// and the same two masks on w >> 8 give (q2,q6) and (q3,q7).  Returns
-// sum_k x_k (q_k + off_k) for the 4 columns, off_k = 1024 (k even) or 64 (k odd).
-__device__ __forceinline__ void unit_fast_int4(const Unit<4, false>& u, const_u32p xw, float acc[4]) {
-    const uint32_t M0 = 0x000F000Fu, M1 = 0x00F000F0u, G0 = 0x64006400u, G1 = 0x54005400u;
+// and the same two masks on w >> 8 give (q2,q6) and (q3,q7).  Staged states per
+// packed row: {x0,x4},{x1,x5},{x2,x6},{x3,x7}.  off_k = 1024 (k even), 64 (k odd).
+// MV_NCOL of the lane's 4 columns are accumulated side by side (independent MFMA
+// chains); fewer chains need fewer accumulator registers at the price of
+// re-reading the staged states.
+#ifndef MV_NCOL
+#define MV_NCOL 2
+#endif
+__device__ __forceinline__ void unit_fast(const Unit<4, false>& u, const h16* xp, f32x4 acc[4]) {
+    const uint32_t M0 = in_vgpr(0x000F000Fu), M1 = in_vgpr(0x00F000F0u);
+    const uint32_t G0 = in_vgpr(0x64006400u), G1 = in_vgpr(0x54005400u);
 #pragma unroll
-    for (int c = 0; c < 4; ++c) acc[c] = 0.f;
+    for (int c0 = 0; c0 < 4; c0 += MV_NCOL) {
 #pragma unroll
-    for (int r = 0; r < 8; ++r) {
-        const uint32_t x01 = xw[4 * r], x23 = xw[4 * r + 1], x45 = xw[4 * r + 2], x67 = xw[4 * r + 3];
-        const uint32_t p04 = pack_lo(x01, x45), p15 = pack_hi(x01, x45);
-        const uint32_t p26 = pack_lo(x23, x67), p37 = pack_hi(x23, x67);
+        for (int r = 0; r < 8; ++r) {
+            const u32x4 p = *reinterpret_cast<const u32x4*>(xp + r * 8);
 #pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            const uint32_t w = u.w[r][c], w8 = w >> 8;
-            acc[c] = dot2((w & M0) | G0, p04, acc[c]);
-            acc[c] = dot2((w & M1) | G1, p15, acc[c]);
-            acc[c] = dot2((w8 & M0) | G0, p26, acc[c]);
-            acc[c] = dot2((w8 & M1) | G1, p37, acc[c]);
+            for (int c = c0; c < c0 + MV_NCOL; ++c) {
+                const uint32_t w = u.w[r][c], w8 = w >> 8;
+                acc[c] = mma4(p.x, p.y, and_or(w, M0, G0), and_or(w, M1, G1), acc[c]);
+                acc[c] = mma4(p.z, p.w, and_or(w8, M0, G0), and_or(w8, M1, G1), acc[c]);
+            }
         }
     }
 }
 
-// Fast int2 path.  Word bits: code j at 2j, 16 codes.  Pairs (j, j+8) share an
-// offset; offsets 0,2,4,6,8 fit the mantissa (magic 2^(10-o)), the remaining
-// codes 5,6,7 / 13,14,15 come down to offsets 0,2,4 after a shift by 10.
-// off_k by k mod 8: 1024, 256, 64, 16, 4, 1024, 256, 64.
-__device__ __forceinline__ void unit_fast_int2(const Unit<2, false>& u, const_u32p xw, float acc[4]) {
-#pragma unroll
-    for (int c = 0; c < 4; ++c) acc[c] = 0.f;
+// int2: word bits: code j at 2j, 16 codes.  Pairs (j, j+8) share an offset;
+// offsets 0,2,4,6,8 fit the mantissa (magic 2^(10-o)); codes 5,6,7 / 13,14,15
+// come down to offsets 0,2,4 after a shift by 10.  Staged states per packed row:
+// {x_j, x_{j+8}} for j = 0..7.  off_k by k mod 8: 1024,256,64,16,4,1024,256,64.
+__device__ __forceinline__ void unit_fast(const Unit<2, false>& u, const h16* xp, f32x4 acc[4]) {
+    const uint32_t M0 = in_vgpr(0x00030003u), M1 = in_vgpr(0x000C000Cu), M2 = in_vgpr(0x00300030u),
+                   M3 = in_vgpr(0x00C000C0u), M4 = in_vgpr(0x03000300u);
+    const uint32_t G0 = in_vgpr(0x64006400u), G1 = in_vgpr(0x5C005C00u), G2 = in_vgpr(0x54005400u),
+                   G3 = in_vgpr(0x4C004C00u), G4 = in_vgpr(0x44004400u);
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-        uint32_t p[8];                                   // p[j] = {x_j, x_{j+8}}
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            const uint32_t a = xw[8 * r + j / 2], b = xw[8 * r + 4 + j / 2];
-            p[j] = (j & 1) ? pack_hi(a, b) : pack_lo(a, b);
-        }
+        const u32x4 pa = *reinterpret_cast<const u32x4*>(xp + r * 16);
+        const u32x4 pb = *reinterpret_cast<const u32x4*>(xp + r * 16 + 8);
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
             const uint32_t w = u.w[r][c], w10 = w >> 10;
-            acc[c] = dot2((w & 0x00030003u) | 0x64006400u, p[0], acc[c]);
-            acc[c] = dot2((w & 0x000C000Cu) | 0x5C005C00u, p[1], acc[c]);
-            acc[c] = dot2((w & 0x00300030u) | 0x54005400u, p[2], acc[c]);
-            acc[c] = dot2((w & 0x00C000C0u) | 0x4C004C00u, p[3], acc[c]);
-            acc[c] = dot2((w & 0x03000300u) | 0x44004400u, p[4], acc[c]);
-            acc[c] = dot2((w10 & 0x00030003u) | 0x64006400u, p[5], acc[c]);
-            acc[c] = dot2((w10 & 0x000C000Cu) | 0x5C005C00u, p[6], acc[c]);
-            acc[c] = dot2((w10 & 0x00300030u) | 0x54005400u, p[7], acc[c]);
+            acc[c] = mma4(pa.x, pa.y, and_or(w, M0, G0), and_or(w, M1, G1), acc[c]);
+            acc[c] = mma4(pa.z, pa.w, and_or(w, M2, G2), and_or(w, M3, G3), acc[c]);
+            acc[c] = mma4(pb.x, pb.y, and_or(w, M4, G4), and_or(w10, M0, G0), acc[c]);
+            acc[c] = mma4(pb.z, pb.w, and_or(w10, M1, G1), and_or(w10, M2, G2), acc[c]);
         }
     }
 }
+__device__ __forceinline__ void unit_fast(const Unit<3, false>&, const h16*, f32x4[4]) {}
+__device__ __forceinline__ void unit_fast(const Unit<4, true>&, const h16*, f32x4[4]) {}
 
-template <int BITS, bool SPARSE> struct FastPath { static constexpr bool HAS = false; };
-template <> struct FastPath<4, false> { static constexpr bool HAS = true; };
-template <> struct FastPath<2, false> { static constexpr bool HAS = true; };
-
-// magic offset of row k (k = index inside the unit) on the fast paths
 template <int BITS>
-__device__ __forceinline__ float fast_offset(int k) {
+__device__ __forceinline__ float fast_offset(int k) {      // magic offset of row k of a unit
     if constexpr (BITS == 4) return (k & 1) ? 64.f : 1024.f;
     const int j = k & 7;
-    const int o = 2 * (j < 5 ? j : j - 5);
-    return (float)(1024 >> o);
+    return (float)(1024 >> (2 * (j < 5 ? j : j - 5)));
 }
 
-// One unit: y[c] += contribution of 64 rows to the lane's 4 columns.
+// ---- general path: any format, either quantisation mode.  Deliberately compact
+// (rolled loops, few registers): it serves the formats without a fast path and
+// the rare exponent-mode columns.  The 32 codes of a block are consumed from a
+// bit stream held in four registers.  States are read in natural order from
+// global memory.  acc[c] = sum over kept k of x_k * value(q_k), xs[c] = sum over
+// kept k of x_k.
 template <int BITS, bool SPARSE>
-__device__ __forceinline__ void process_unit(const Unit<BITS, SPARSE>& u, const MatvecArgs& a,
-                                             int unit, int lane, float y[4]) {
-    const_u32p xw = to_const(a.x) + unit * 32;           // 64 halves, wave-uniform
-    const h16x2 s01 = as_h2(u.sc.x), s23 = as_h2(u.sc.y);
-    const h16x2 z01 = as_h2(u.ze.x), z23 = as_h2(u.ze.y);
-    const float sc[4] = {(float)s01.x, (float)s01.y, (float)s23.x, (float)s23.y};
-    const float ze[4] = {(float)z01.x, (float)z01.y, (float)z23.x, (float)z23.y};
-    const bool expo[4] = {!(sc[0] >= 0.f), !(sc[1] >= 0.f), !(sc[2] >= 0.f), !(sc[3] >= 0.f)};
-    const bool any_expo = __builtin_amdgcn_ballot_w64(expo[0] | expo[1] | expo[2] | expo[3]) != 0;
-
-    const float xsum = SPARSE ? 0.f : wave_sum(u.xl);    // sum of the unit's 64 states
-    float acc[4], xs[4];
-    bool fast = false;
-    if constexpr (FastPath<BITS, SPARSE>::HAS) {
-        if (!any_expo) {
-            fast = true;
-            const float off = wave_sum(u.xl * fast_offset<BITS>(lane));
-            if constexpr (BITS == 4) unit_fast_int4(u, xw, acc);
-            else unit_fast_int2(u, xw, acc);
-#pragma unroll
-            for (int c = 0; c < 4; ++c) acc[c] -= off;
-        }
-    }
-    if (!fast) unit_generic<BITS, SPARSE>(u, xw, expo, acc, xs);
+__device__ __forceinline__ void unit_generic(const Unit<BITS, SPARSE>& u, const h16* __restrict__ xg,
+                                             const bool expo[4], float acc[4], float xs[4]) {
+    constexpr int WPB = SPARSE ? 2 : BITS;           // packed words per 32-row block
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
-        const float xc = SPARSE ? xs[c] : xsum;
-        // linear: s * (acc - z * X)      exponent: (-s) * acc + z * X
-        const float lin = sc[c] * (acc[c] - ze[c] * xc);
-        const float ex = ze[c] * xc - sc[c] * acc[c];
-        y[c] += expo[c] ? ex : lin;
+        float ac = 0.f, xc = 0.f;
+#pragma unroll
+        for (int hb = 0; hb < 2; ++hb) {
+            uint32_t s[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+            for (int i = 0; i < WPB; ++i) s[i] = u.w[hb * WPB + i][c];
+            uint32_t keep = 0xFFFFFFFFu;
+            if constexpr (SPARSE) keep = u.m[hb][c];
+#pragma unroll 2
+            for (int t = 0; t < 32; ++t) {
+                const uint32_t code = s[0] & ((1u << BITS) - 1u);
+                const bool k = keep & 1u;
+                keep >>= 1;
+                const uint32_t sh = SPARSE ? (k ? 4u : 0u) : (uint32_t)BITS;
+                s[0] = __builtin_amdgcn_alignbit(s[1], s[0], sh);
+                s[1] = __builtin_amdgcn_alignbit(s[2], s[1], sh);
+                s[2] = __builtin_amdgcn_alignbit(s[3], s[2], sh);
+                s[3] >>= sh;
+                const float xv = (float)xg[hb * 32 + t];
+                const float val = code_value<BITS>(code, expo[c]);
+                ac += k ? xv * val : 0.f;
+                xc += k ? xv : 0.f;
+            }
+        }
+        acc[c] = ac;
+        xs[c] = xc;
     }
 }
 
-template <int BITS, bool SPARSE>
-__global__ __launch_bounds__(MV_MAX_WAVES * WAVE) void matvec_kernel(MatvecArgs a) {
-    __shared__ float red[MV_MAX_WAVES][MV_COLS];
-    __shared__ int is_last;
+__device__ __forceinline__ void unpack_params(const u32x2 sc2, const u32x2 ze2, float sc[4], float ze[4],
+                                              bool expo[4]) {
+    const h16x2 s01 = as_h2(sc2.x), s23 = as_h2(sc2.y), z01 = as_h2(ze2.x), z23 = as_h2(ze2.y);
+    sc[0] = (float)s01.x; sc[1] = (float)s01.y; sc[2] = (float)s23.x; sc[3] = (float)s23.y;
+    ze[0] = (float)z01.x; ze[1] = (float)z01.y; ze[2] = (float)z23.x; ze[3] = (float)z23.y;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) expo[c] = !(sc[c] >= 0.f);     // NaN takes the exponent branch
+}
 
-    const int lane = threadIdx.x & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int nwaves = blockDim.x >> 6;
+// sum over an aligned group of 4 / 8 lanes (valid in every lane of the group)
+__device__ __forceinline__ float sum4(float v) {
+    v += dpp_f32<0xB1>(v);
+    v += dpp_f32<0x4E>(v);
+    return v;
+}
+__device__ __forceinline__ float sum8(float v) {
+    v += dpp_f32<0xB1>(v);
+    v += dpp_f32<0x4E>(v);
+    v += dpp_f32<0x141>(v);
+    return v;
+}
+
+// ---- cross-workgroup hand-over.  A slot is 8 bytes {fp32 partial sum, flag};
+// it is written with one device-scope (write-through) 64-bit store and read
+// with device-scope loads, so no cache-wide fence is needed and a writer never
+// waits.  flag == SLOT_FULL marks a slot as written; the reader clears it.
+constexpr uint32_t SLOT_FULL = 0x600DF00Du;
+constexpr int MV_SPIN_LIMIT = 1 << 22;            // polls before a reader gives up
+
+__device__ __forceinline__ void slot_store(uint64_t* p, float v, uint32_t flag) {
+    const uint64_t bits = (uint64_t)bitcast<uint32_t>(v) | ((uint64_t)flag << 32);
+    __hip_atomic_store(p, bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ uint64_t slot_load(const uint64_t* p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// PF: keep the next unit's loads in flight while the current one is processed
+// (more registers); without it a lane group loads and processes one unit at a
+// time and relies on the other resident waves to cover the latency.
+template <int BITS, bool SPARSE, int LK, bool PF>
+__global__ __launch_bounds__(MV_MAX_WAVES * WAVE)
+void matvec_kernel(MatvecArgs a) {
+    constexpr bool FAST = Fmt<BITS, SPARSE>::FAST;
+    constexpr int LC = WAVE / LK;                 // column lanes per lane group
+    constexpr int COLS = LC * 4;                  // columns per strip
+
+    // staged states (64 halves per unit) then per-unit {sum x, sum off*x}; the
+    // same memory is reused for the final reduction
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    h16* xs = reinterpret_cast<h16*>(smem);
+    float* sums = reinterpret_cast<float*>(smem + (size_t)a.units_per_wg * 128);
+    float* red = reinterpret_cast<float*>(smem);
+
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6, nwaves = blockDim.x >> 6;
+    const int cl = lane % LC, kl = lane / LC;
     const int strip = blockIdx.x, split = blockIdx.y;
-    const int col = strip * MV_COLS + lane * 4;
+    const int col = strip * COLS + cl * 4;
     const bool col_ok = col < a.S;
 
-    const int u_begin = (split * nwaves + wave) * a.units_per_wave;
-    const int u_end = min(u_begin + a.units_per_wave, a.units_total);
+    const int wg_u0 = split * a.units_per_wg;
+    const int wg_u1 = min(wg_u0 + a.units_per_wg, a.units_total);
+    const int ng = nwaves * LK, grp = wave * LK + kl;
+
+    // ---- issue order matters: loads return in order, so the (small) loads of
+    // the states go first and the weight loads follow; the staging below then
+    // only waits for the states while the weights are still in flight.
+    constexpr int HPR = BITS == 2 ? 16 : 8;       // halves (k values) per staged row
+    constexpr int RPU = 64 / HPR;                 // staged rows per unit
+    const int nrows = FAST ? (wg_u1 - wg_u0) * RPU : 0;
+    const int nrows8 = (nrows + 7) & ~7;
+    const h16* xg = a.x + wg_u0 * 64;
+    u32x4 xa = {0, 0, 0, 0}, xb = {0, 0, 0, 0};
+    auto load_x = [&](int r) {
+        if (r < nrows) {
+            xa = *reinterpret_cast<const u32x4*>(xg + r * HPR);
+            if constexpr (HPR == 16) xb = *reinterpret_cast<const u32x4*>(xg + r * HPR + 8);
+        }
+    };
+    if constexpr (FAST) load_x(t);
+
+    Unit<BITS, SPARSE> ua, ub;
+    int u = wg_u0 + grp;
+    const bool work = col_ok && u < wg_u1;
+    const bool work_b = PF && work && u + ng < wg_u1;
+    if (work) load_unit(ua, a, u, col);
+    if constexpr (PF) {
+        if (work_b) load_unit(ub, a, u + ng, col);
+    }
+
+    if constexpr (FAST) {
+        for (int r = t; r < nrows8; r += blockDim.x) {
+            if (r != t) load_x(r);
+            float s = 0.f, o = 0.f;
+            if (r < nrows) {
+                if constexpr (BITS == 4) {
+                    const u32x4 v = xa;                                           // x0x1 x2x3 x4x5 x6x7
+                    u32x4 p;
+                    p.x = __builtin_amdgcn_perm(v.z, v.x, 0x05040100u);            // {x0, x4}
+                    p.y = __builtin_amdgcn_perm(v.z, v.x, 0x07060302u);            // {x1, x5}
+                    p.z = __builtin_amdgcn_perm(v.w, v.y, 0x05040100u);            // {x2, x6}
+                    p.w = __builtin_amdgcn_perm(v.w, v.y, 0x07060302u);            // {x3, x7}
+                    *reinterpret_cast<u32x4*>(xs + r * 8) = p;
+                    const float e = lo_f32(v.x) + lo_f32(v.y) + lo_f32(v.z) + lo_f32(v.w);
+                    const float d = hi_f32(v.x) + hi_f32(v.y) + hi_f32(v.z) + hi_f32(v.w);
+                    s = e + d;
+                    o = 1024.f * e + 64.f * d;
+                } else {
+                    const u32x4 va = xa, vb = xb;
+                    u32x4 pa, pb;
+                    pa.x = __builtin_amdgcn_perm(vb.x, va.x, 0x05040100u);         // {x0, x8}
+                    pa.y = __builtin_amdgcn_perm(vb.x, va.x, 0x07060302u);         // {x1, x9}
+                    pa.z = __builtin_amdgcn_perm(vb.y, va.y, 0x05040100u);
+                    pa.w = __builtin_amdgcn_perm(vb.y, va.y, 0x07060302u);
+                    pb.x = __builtin_amdgcn_perm(vb.z, va.z, 0x05040100u);
+                    pb.y = __builtin_amdgcn_perm(vb.z, va.z, 0x07060302u);
+                    pb.z = __builtin_amdgcn_perm(vb.w, va.w, 0x05040100u);
+                    pb.w = __builtin_amdgcn_perm(vb.w, va.w, 0x07060302u);
+                    *reinterpret_cast<u32x4*>(xs + r * 16) = pa;
+                    *reinterpret_cast<u32x4*>(xs + r * 16 + 8) = pb;
+                    const uint32_t w[8] = {va.x, va.y, va.z, va.w, vb.x, vb.y, vb.z, vb.w};
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) {
+                        const float lo = lo_f32(w[j]), hi = hi_f32(w[j]);
+                        s += lo + hi;
+                        o += lo * fast_offset<2>(2 * j) + hi * fast_offset<2>(2 * j + 1);
+                    }
+                }
+            }
+            if constexpr (RPU == 8) { s = sum8(s); o = sum8(o); }
+            else { s = sum4(s); o = sum4(o); }
+            if ((r % RPU) == 0 && r < nrows) {     // first row of a unit publishes its sums
+                sums[(r / RPU) * 2] = s;
+                sums[(r / RPU) * 2 + 1] = o;
+            }
+        }
+        __syncthreads();
+    }
 
     float y[4] = {0.f, 0.f, 0.f, 0.f};
-    if (u_begin < u_end) {
-        Unit<BITS, SPARSE> ua, ub;
-        load_unit(ua, a, u_begin, col, col_ok, lane);
-        for (int u = u_begin; u < u_end; u += 2) {
-            const bool has_b = u + 1 < u_end;
-            if (has_b) load_unit(ub, a, u + 1, col, col_ok, lane);
-            process_unit(ua, a, u, lane, y);
-            if (has_b) {
-                if (u + 2 < u_end) load_unit(ua, a, u + 2, col, col_ok, lane);
-                process_unit(ub, a, u + 1, lane, y);
+    bool need_general = false;
+
+    auto finish_unit = [&](const Unit<BITS, SPARSE>& un, int unit) {
+        float sc[4], ze[4];
+        bool expo[4];
+        unpack_params(un.sc, un.ze, sc, ze, expo);
+        if constexpr (FAST) {
+            f32x4 acc[4];
+#pragma unroll
+            for (int c = 0; c < 4; ++c) acc[c] = f32x4{0.f, 0.f, 0.f, 0.f};
+            const int lu = unit - wg_u0;
+            unit_fast(un, xs + lu * 64, acc);
+            const float xsum = sums[lu * 2], xoff = sums[lu * 2 + 1];
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                // exponent-mode columns (scale < 0 or NaN) contribute nothing here
+                const float sl = fmaxf(sc[c], 0.f);
+                y[c] += sl * ((acc[c][0] - xoff) - ze[c] * xsum);
+                need_general |= expo[c];
+            }
+        } else {
+            float acc[4], xsv[4];
+            unit_generic<BITS, SPARSE>(un, a.x + unit * 64, expo, acc, xsv);
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const float lin = sc[c] * (acc[c] - ze[c] * xsv[c]);
+                const float ex = ze[c] * xsv[c] - sc[c] * acc[c];
+                y[c] += expo[c] ? ex : lin;
+            }
+        }
+    };
+
+    if (work) {
+        if constexpr (PF) {
+            // ua and ub are both in flight on entry
+            bool has_b = work_b;
+            for (;;) {
+                finish_unit(ua, u);
+                if (!has_b) break;
+                const int u2 = u + 2 * ng, u3 = u + 3 * ng;
+                const bool has_a = u2 < wg_u1;
+                if (has_a) load_unit(ua, a, u2, col);
+                finish_unit(ub, u + ng);
+                if (!has_a) break;
+                has_b = u3 < wg_u1;
+                if (has_b) load_unit(ub, a, u3, col);
+                u = u2;
+            }
+        } else {
+            for (;;) {
+                finish_unit(ua, u);
+                u += ng;
+                if (u >= wg_u1) break;
+                load_unit(ua, a, u, col);
             }
         }
     }
 
-    // ---- workgroup reduction through LDS
-    *reinterpret_cast<f32x4*>(&red[wave][lane * 4]) = f32x4{y[0], y[1], y[2], y[3]};
-    __syncthreads();
-    const int t = threadIdx.x;
-    float total = 0.f;
-    const int ocol = strip * MV_COLS + t;
-    const bool owner = t < MV_COLS && ocol < a.S;
-    if (owner) {
-        for (int w = 0; w < nwaves; ++w) total += red[w][t];
+    if constexpr (FAST) {
+        // exponent-mode columns: second pass with the general decoder, only where needed
+        if (__builtin_amdgcn_ballot_w64(need_general) != 0 && work) {
+            for (int v = wg_u0 + grp; v < wg_u1; v += ng) {
+                load_unit(ua, a, v, col);
+                float sc[4], ze[4], acc[4], xsv[4];
+                bool expo[4];
+                unpack_params(ua.sc, ua.ze, sc, ze, expo);
+                if (!(expo[0] | expo[1] | expo[2] | expo[3])) continue;
+                unit_generic<BITS, SPARSE>(ua, a.x + v * 64, expo, acc, xsv);
+#pragma unroll
+                for (int c = 0; c < 4; ++c) y[c] += expo[c] ? ze[c] * xsv[c] - sc[c] * acc[c] : 0.f;
+            }
+        }
     }
+
+    // ---- workgroup reduction through LDS (the staging area is free now)
+    __syncthreads();
+    *reinterpret_cast<f32x4*>(&red[(wave * 64 + lane) * 4]) = f32x4{y[0], y[1], y[2], y[3]};
+    __syncthreads();
+    // each thread finishes the columns j = t, t + blockDim.x, ... of the strip
+    // (a workgroup may have fewer threads than the strip has columns)
+    constexpr int MAXC = COLS / WAVE;                      // columns per thread with one wave
+    float total[MAXC];
+#pragma unroll
+    for (int i = 0; i < MAXC; ++i) {
+        const int j = t + i * (int)blockDim.x;
+        total[i] = 0.f;
+        if (j < COLS) {
+            for (int w = 0; w < nwaves; ++w)
+#pragma unroll
+                for (int k = 0; k < LK; ++k) total[i] += red[(w * 64 + k * LC) * 4 + j];
+        }
+    }
+    auto for_owned = [&](auto&& fn) {
+#pragma unroll
+        for (int i = 0; i < MAXC; ++i) {
+            const int j = t + i * (int)blockDim.x;
+            const int ocol = strip * COLS + j;
+            if (j < COLS && ocol < a.S) fn(i, ocol);
+        }
+    };
     if (a.splits == 1) {
-        if (owner) a.outs[ocol] = (h16)((float)a.outs[ocol] + total);
+        for_owned([&](int i, int ocol) { a.outs[ocol] = (h16)((float)a.outs[ocol] + total[i]); });
         return;
     }
 
-    // ---- across workgroups: fp32 slot per split, last arrival finishes
-    if (owner) a.partials[(int64_t)split * a.S + ocol] = total;
-    __threadfence();
-    __syncthreads();
-    if (t == 0) {
-        const int prev = __hip_atomic_fetch_add(&a.counters[strip], 1, __ATOMIC_ACQ_REL,
-                                                __HIP_MEMORY_SCOPE_AGENT);
-        is_last = prev == a.splits - 1;
+    // ---- across workgroups.  Splits 0 .. n-2 publish their partial sums and
+    // leave.  Split n-1 has the highest workgroup index of its strip, so by the
+    // time it runs every other split has been dispatched: it waits for their
+    // slots, adds them in a fixed order (deterministic), clears them for the
+    // next call and writes the result.
+    if (split != a.splits - 1) {
+        for_owned([&](int i, int ocol) { slot_store(&a.slots[(int64_t)split * a.S + ocol], total[i], SLOT_FULL); });
+        return;
     }
-    __syncthreads();
-    if (!is_last) return;
-    __threadfence();
-    if (owner) {
-        float sum = 0.f;
-        for (int sp = 0; sp < a.splits; ++sp)
-            sum += __builtin_nontemporal_load(&a.partials[(int64_t)sp * a.S + ocol]);
-        a.outs[ocol] = (h16)((float)a.outs[ocol] + sum);
-    }
-    if (t == 0) a.counters[strip] = 0;                    // ready for the next call
+    for_owned([&](int i, int ocol) {
+        float sum = (float)a.outs[ocol];
+        bool ok = true;
+        // slots are fetched eight at a time so that their latencies overlap; a
+        // slot that is not full yet is polled again on its own
+        for (int s0 = 0; s0 < a.splits - 1; s0 += 8) {
+            uint64_t v[8];
+#pragma unroll
+            for (int k = 0; k < 8; ++k)
+                v[k] = s0 + k < a.splits - 1 ? slot_load(&a.slots[(int64_t)(s0 + k) * a.S + ocol]) : 0;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                if (s0 + k >= a.splits - 1) break;
+                uint64_t* p = &a.slots[(int64_t)(s0 + k) * a.S + ocol];
+                int spins = 0;
+                while ((uint32_t)(v[k] >> 32) != SLOT_FULL && spins < MV_SPIN_LIMIT) {
+                    __builtin_amdgcn_s_sleep(1);
+                    v[k] = slot_load(p);
+                    ++spins;
+                }
+                ok &= (uint32_t)(v[k] >> 32) == SLOT_FULL;
+                sum += bitcast<float>((uint32_t)v[k]);
+                slot_store(p, 0.f, 0u);
+            }
+        }
+        sum += total[i];
+        // a slot that never arrived (which would mean a writer was never run)
+        // poisons the output instead of hanging the wave
+        a.outs[ocol] = ok ? (h16)sum : (h16)__builtin_nanf("");
+    });
 }
 
 template <int BITS, bool SPARSE>
-static void launch(const MatvecArgs& a, dim3 grid, dim3 block, hipStream_t st) {
-    hipLaunchKernelGGL((matvec_kernel<BITS, SPARSE>), grid, block, 0, st, a);
+static void launch(const MatvecArgs& a, int lk, bool pf, dim3 grid, dim3 block, size_t lds, hipStream_t st) {
+#define I4_LAUNCH(LK_, PF_) hipLaunchKernelGGL((matvec_kernel<BITS, SPARSE, LK_, PF_>), grid, block, lds, st, a)
+    if (lk == 1) { if (pf) I4_LAUNCH(1, true); else I4_LAUNCH(1, false); }
+    else if (lk == 2) { if (pf) I4_LAUNCH(2, true); else I4_LAUNCH(2, false); }
+    else { if (pf) I4_LAUNCH(4, true); else I4_LAUNCH(4, false); }
+#undef I4_LAUNCH
 }
 
 }  // namespace i4
@@ -343,57 +525,66 @@ extern "C" int int4mm_matvec(int bits, void* outs, const void* matrix, const voi
     if (B * shape->seq_len * S == 0) return INT4MM_OK;
 
     const int units_total = (int)(K / 64);
-    const int strips = (int)((S + MV_COLS - 1) / MV_COLS);
     const int64_t g = shape->group_size < 0 ? ONE_GROUP : shape->group_size;
 
-    // Work split: aim for ~16 resident waves on each of the 256 CUs.
-    int waves = (int)tuning(TUNE_MV_WAVES), upw = (int)tuning(TUNE_MV_UNITS);
-    if (upw <= 0) {
-        const int64_t want_waves = 256 * 12;
-        int64_t per_strip = (want_waves + strips - 1) / strips;
-        upw = (int)((units_total + per_strip - 1) / per_strip);
-        if (upw < 1) upw = 1;
+    // Launch shape: strips of 256/lk columns, `waves` waves per workgroup, `upwg`
+    // units per workgroup dealt round-robin to its lane groups; the grid's y
+    // dimension covers the rest of K.
+    // Defaults (measured on MI355X): the narrowest lane-group split that still
+    // gives about 160 strips, about 640 workgroups in all (2.5 per CU, all
+    // resident at once), 4 waves each.
+    int lk = (int)tuning(TUNE_MV_LK), waves = (int)tuning(TUNE_MV_WAVES), upwg = (int)tuning(TUNE_MV_UNITS);
+    if (lk != 1 && lk != 2 && lk != 4) {
+        lk = 1;
+        while (lk < 4 && (S + 256 / lk - 1) / (256 / lk) < 160) lk *= 2;
     }
+    const int cols = 256 / lk;
+    const int strips = (int)((S + cols - 1) / cols);
     if (waves <= 0) waves = 4;
     if (waves > MV_MAX_WAVES) waves = MV_MAX_WAVES;
-    int runs = (units_total + upw - 1) / upw;             // wave-sized runs along K
-    if (waves > runs) waves = runs;
-    int splits = (runs + waves - 1) / waves;
-    if (splits > MV_MAX_SPLITS) {                          // keep the slot count bounded
-        splits = MV_MAX_SPLITS;
-        upw = (units_total + splits * waves - 1) / (splits * waves);
-        runs = (units_total + upw - 1) / upw;
-        splits = (runs + waves - 1) / waves;
+    if (upwg <= 0) {
+        int want_splits = (640 + strips / 2) / strips;
+        if (want_splits < 1) want_splits = 1;
+        upwg = (units_total + want_splits - 1) / want_splits;
+        if (upwg < 4) upwg = 4;
     }
-    if (splits > 1) {
-        if (workspace == nullptr || workspace_bytes < int4mm_workspace_bytes(S))
-            return INT4MM_ERR_WORKSPACE;
-        if (strips * 4 > 4096) return INT4MM_ERR_SHAPE;
+    if (upwg > units_total) upwg = units_total;
+    int splits = (units_total + upwg - 1) / upwg;
+    if (splits > MV_MAX_SPLITS) {                           // bounded slot count: more units each
+        upwg = (units_total + MV_MAX_SPLITS - 1) / MV_MAX_SPLITS;
+        splits = (units_total + upwg - 1) / upwg;
     }
+    if (waves * lk > upwg) waves = (upwg + lk - 1) / lk;    // no idle waves
+    if (upwg > MV_MAX_UNITS_WG) return INT4MM_ERR_SHAPE;
+    if (splits > 1 && (workspace == nullptr || workspace_bytes < int4mm_workspace_bytes(S)))
+        return INT4MM_ERR_WORKSPACE;
+    // software prefetch only pays when lane groups walk several units
+    const bool pf = upwg >= 3 * waves * lk && tuning(TUNE_MV_NOPF) == 0;
 
     MatvecArgs a;
     a.matrix = (const uint32_t*)matrix;
     a.mask = (const uint32_t*)sparse_mask;
     a.scales = (const h16*)scales;
     a.zeros = (const h16*)zeros;
-    a.counters = (int*)workspace;
-    a.partials = workspace ? (float*)((char*)workspace + 4096) : nullptr;
+    a.slots = (uint64_t*)workspace;
     a.K = (int)K;
     a.S = (int)S;
     a.units_total = units_total;
-    a.units_per_wave = upw;
+    a.units_per_wg = upwg;
     a.group_units = (int)(g / 64 > 0x7FFFFFF ? 0x7FFFFFF : g / 64);
     a.splits = splits;
 
+    size_t lds = (size_t)upwg * 136;
+    if (lds < (size_t)waves * 1024) lds = (size_t)waves * 1024;
     const dim3 grid(strips, splits, 1), block(waves * WAVE);
     hipStream_t st = (hipStream_t)stream;
     for (int64_t b = 0; b < B; ++b) {                      // one pass over the weights per batch row
         a.outs = (h16*)outs + b * S;
         a.x = (const h16*)multiplier + b * K;
-        if (sparse_mask) launch<4, true>(a, grid, block, st);
-        else if (bits == 4) launch<4, false>(a, grid, block, st);
-        else if (bits == 3) launch<3, false>(a, grid, block, st);
-        else launch<2, false>(a, grid, block, st);
+        if (sparse_mask) launch<4, true>(a, lk, pf, grid, block, lds, st);
+        else if (bits == 4) launch<4, false>(a, lk, pf, grid, block, lds, st);
+        else if (bits == 3) launch<3, false>(a, lk, pf, grid, block, lds, st);
+        else launch<2, false>(a, lk, pf, grid, block, lds, st);
         rc = check_launch("matvec");
         if (rc != INT4MM_OK) return rc;
     }
