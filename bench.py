@@ -1,0 +1,185 @@
+#!/usr/bin/env python3
+"""Headline benchmark: int4 x fp16 matvec at K(N)=5120, S=20480, M=1, g=128 on one
+MI355X, through the C ABI of libint4mm_hip.so.
+
+A step is one matvec over one set of packed weights.  Seven distinct weight sets
+(390 MB, more than the 256 MB last-level cache) are used in rotation so that
+every step streams its weights from HBM.  The timed region is K steps captured
+in one HIP graph (no host work between kernels), bracketed by synchronisation;
+HIP events recorded on the launch stream around the same region give the average
+kernel duration used for the roofline figure.  The int4 matmul at M=2048 is
+measured the same way and reported beside it, and the torch-CPU
+dequantise-then-matmul baseline is timed on the host on a bounded sample.
+
+Prints ONE JSON line.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
+MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 MFMA
+
+# HBM bytes per matvec launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see
+# profiles/); None until measured
+MATVEC_TRAFFIC_BYTES = None
+
+
+def matvec_bytes(K, S, g, bits=4):
+    return K * bits // 32 * S * 4 + 2 * (K // g) * S * 2 + 2 * K + 2 * S
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=700)
+    ap.add_argument("--warmup", type=int, default=50)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-gemm", action="store_true", help="skip the M=2048 matmul leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (the matvec/matmul shard "
+              "by output columns without any exchange); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+
+    from int4matmul_kernels_amd import capi
+    from oracle import oracle as O
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = "cuda:0"
+    torch.cuda.set_device(0)
+    K, S, g, NSETS = 5120, 20480, 128, 7
+    steps, warmup = max(1, args.steps), max(0, args.warmup)
+
+    # ---- seeded synthetic workload (BASELINE config 2); set 0 is the oracle's problem
+    p = O.make_problem(K=K, S=S, M=1, bits=4, group_size=g, seed=0)
+    gen = torch.Generator(device="cpu").manual_seed(0)
+    sets = []
+    for i in range(NSETS):
+        if i == 0:
+            m, sc, ze = (torch.from_numpy(p["matrix"]), torch.from_numpy(p["scales"]), torch.from_numpy(p["zeros"]))
+        else:
+            m = torch.randint(-2 ** 31, 2 ** 31 - 1, (K // 8, S), dtype=torch.int32, generator=gen)
+            sc = torch.empty((K // g, S)).uniform_(0.001, 0.02, generator=gen).half()
+            ze = torch.empty((K // g, S)).uniform_(0.0, 15.0, generator=gen).half()
+        sets.append((m.to(dev), sc.to(dev), ze.to(dev)))
+    x = torch.from_numpy(p["states"]).to(dev)
+    xneg = -x                                   # alternate sign so that outs does not grow
+    outs = [torch.zeros((1, 1, S), dtype=torch.float16, device=dev) for _ in range(NSETS)]
+    ws = capi.new_workspace(S)
+
+    def step(i):
+        m, sc, ze = sets[i % NSETS]
+        xi = x if (i // NSETS) % 2 == 0 else xneg
+        capi.matvec(4, outs[i % NSETS], m, xi, sc, ze, g, None, ws)
+
+    # ---- correctness of the measured path against the oracle (set 0, fresh outs)
+    chk = torch.zeros((1, 1, S), dtype=torch.float16, device=dev)
+    capi.matvec(4, chk, sets[0][0], x, sets[0][1], sets[0][2], g, None, ws)
+    torch.cuda.synchronize()
+    w32 = O.dequantize_matrix_fp32(4, p["matrix"], p["scales"], p["zeros"], g)
+    want = O.matmul_fp32(p["states"][0], w32)
+    err = O.max_rel_error(want, chk.cpu().numpy()[0])
+    assert err < 1e-2, f"matvec disagrees with the oracle: max relative error {err}"
+
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        for i in range(warmup):
+            step(i)
+        stream.synchronize()
+        # K steps in one graph: back-to-back kernels, no host work in the timed region
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            for i in range(steps):
+                step(i)
+        graph.replay()                            # untimed: first replay uploads the graph
+        stream.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        e0.record(stream)
+        graph.replay()
+        e1.record(stream)
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+    wall_s = t1 - t0
+    ev_us = e0.elapsed_time(e1) * 1e3 / steps     # average launch duration, HIP events on the launch stream
+    nbytes = matvec_bytes(K, S, g)
+    value = nbytes * steps / wall_s / 1e9
+    achieved = nbytes / (ev_us * 1e-6) / 1e9
+
+    result = {
+        "metric": "int4 GEMV GB/s & us (N=5120,S=20480,M=1); int4 GEMM TFLOP/s at M=2048",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+        "ms_per_step": wall_s * 1e3 / steps, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "fp16", "data": "synthetic",
+        "config": {"workload": "int4 dense matvec K(N)=5120 S=20480 M=1 B=1 group=128, "
+                               f"{NSETS} weight sets in rotation (cold HBM)",
+                   "bytes_per_step": nbytes, "us_per_step": round(wall_s * 1e6 / steps, 3),
+                   "max_rel_err_vs_fp32_oracle": float(f"{err:.3e}")},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MATVEC_TRAFFIC_BYTES,
+                     "kernel": "i4::matvec_kernel<4,false,...>", "avg_launch_us": round(ev_us, 3)},
+    }
+
+    # ---- the matmul half of the metric: M=2048, same weights (BASELINE config 3)
+    if not args.no_gemm:
+        M = 2048
+        xs = torch.randn((1, M, K), generator=torch.Generator(device="cpu").manual_seed(1)).half().to(dev)
+        om = torch.zeros((1, M, S), dtype=torch.float16, device=dev)
+        m, sc, ze = sets[0]
+        with torch.cuda.stream(stream):
+            for _ in range(3):
+                capi.matmul(4, om, m, xs, sc, ze, g, None, ws)
+            stream.synchronize()
+            reps = 20
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            for _ in range(reps):
+                capi.matmul(4, om, m, xs, sc, ze, g, None, ws)
+            e1.record(stream)
+            stream.synchronize()
+        mm_us = e0.elapsed_time(e1) * 1e3 / reps
+        flops = 2.0 * M * K * S
+        tf = flops / (mm_us * 1e-6) / 1e12
+        # spot check: 16 rows against the fp32 oracle
+        rows = np.linspace(0, M - 1, 16).astype(int)
+        got = om[0, rows].cpu().numpy()
+        want_mm = O.matmul_fp32(xs[0, rows].cpu().numpy(), w32)
+        mm_err = O.max_rel_error(want_mm, got)
+        assert mm_err < 1e-2, f"matmul disagrees with the oracle: {mm_err}"
+        result["gemm"] = {"workload": "int4 dense matmul M=2048 K(N)=5120 S=20480 group=128",
+                          "us": round(mm_us, 2), "tflops": round(tf, 1),
+                          "roofline": {"bound": "mfma", "achieved": round(tf, 1), "peak": MFMA_FP16_PEAK_TFLOPS,
+                                       "unit": "TFLOP/s", "frac": round(tf / MFMA_FP16_PEAK_TFLOPS, 4),
+                                       "traffic": None},
+                          "max_rel_err_vs_fp32_oracle": float(f"{mm_err:.3e}")}
+
+    # ---- CPU baseline: torch dequantise + fp32 matmul on the host (reported only)
+    if not args.no_cpu:
+        from oracle import cpu_baseline
+
+        r = cpu_baseline.time_matvec(p, budget_s=15.0)
+        cpu_err = O.max_rel_error(want, r["result"])
+        result["cpu_baseline"] = {
+            "value": round(nbytes / r["best_s"] / 1e9, 3), "unit": "GB/s", "cores": r["threads"], "kind": "port",
+            "sample": f"the full K=5120 S=20480 matvec, best of {r['reps']} repetitions "
+                      f"(dequantise {r['dequant_s'] * 1e3:.0f} ms + fp32 matmul {r['matmul_s'] * 1e3:.1f} ms)",
+            "us_per_step": round(r["best_s"] * 1e6, 1), "host_cpus": os.cpu_count(),
+            "max_rel_err_vs_fp32_oracle": float(f"{cpu_err:.3e}")}
+
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()
