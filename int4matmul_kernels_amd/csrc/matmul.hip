@@ -5,15 +5,22 @@
 //
 // One workgroup owns a BM x BN tile of outs and walks K in steps of 64.  Per
 // step the packed weights of the tile (64 x BN codes) are read from HBM once,
-// decoded and dequantised to fp16 ONCE by the workgroup (2 threads per column,
-// one 32-row block each) and stored to LDS in the operand layout of
-// v_mfma_f32_32x32x16_f16: 16-byte chunks of 8 consecutive k for one column,
-// chunk (kc, n) at kc*BN + n, which both the writes (lanes along n) and the MFMA
-// operand reads (lanes along n) touch without bank conflicts.  The states tile
-// (BM x 64 fp16) is stored row-major with an XOR swizzle of the chunk index so
-// that row-contiguous writes and column-of-rows operand reads are both
-// conflict-free.  Accumulation is fp32 in the MFMA accumulators.
+// decoded and dequantised to fp16 ONCE by the workgroup and stored to LDS in
+// the operand layout of v_mfma_f32_32x32x16_f16: 16-byte chunks of 8
+// consecutive k for one column, chunk (kc, n) at kc*BN + n, which both the
+// writes (lanes along n) and the MFMA operand reads (lanes along n) touch
+// without bank conflicts.  The states tile (BM x 64 fp16) is stored row-major
+// with an XOR swizzle of the chunk index so that row-contiguous writes and
+// column-of-rows operand reads are both conflict-free.  Accumulation is fp32 in
+// the MFMA accumulators.  Global loads of step k+1 are issued before the MFMA
+// phase of step k (register prefetch); two workgroups share a CU so that one
+// decodes while the other multiplies.
+//
+// Workgroups are renumbered so that the 8 XCDs (each with its own L2) take
+// disjoint column ranges of the weight matrix.
 #include "common.h"
+
+#include <type_traits>
 
 namespace i4 {
 
@@ -31,6 +38,7 @@ struct MatmulArgs {
     const h16* zeros;
     int M, K, S;
     int group_units;        // group size / 64
+    int tiles_m, tiles_n;
 };
 
 // Raw packed data of one (32-row block, column) cell
@@ -38,7 +46,6 @@ template <int BITS, bool SPARSE>
 struct Cell {
     uint32_t w[SPARSE ? 2 : BITS];
     uint32_t m;
-    h16 sc, ze;
 };
 
 template <int BITS, bool SPARSE>
@@ -49,14 +56,12 @@ __device__ __forceinline__ void load_cell(Cell<BITS, SPARSE>& c, const MatmulArg
 #pragma unroll
     for (int r = 0; r < ROWS; ++r) c.w[r] = p[r * S];
     c.m = SPARSE ? a.mask[(int64_t)blk * S + col] : 0xFFFFFFFFu;
-    const int64_t gofs = (int64_t)((blk >> 1) / a.group_units) * S + col;
-    c.sc = a.scales[gofs];
-    c.ze = a.zeros[gofs];
 }
 
-// Cell -> 32 fp16 weights = 4 chunks of 8, bit-exact with the reference decode
+// General cell decode: 32 fp16 weights = 4 chunks of 8, bit-exact with the
+// reference decode, any format and either quantisation mode.
 template <int BITS, bool SPARSE>
-__device__ __forceinline__ void dequant_cell(const Cell<BITS, SPARSE>& c, h16x8 out[4]) {
+__device__ __forceinline__ void dequant_cell_generic(const Cell<BITS, SPARSE>& c, h16 sc, h16 ze, h16x8 out[4]) {
     uint32_t codes[32];
     if constexpr (SPARSE) {
         uint64_t v = (uint64_t)c.w[0] | ((uint64_t)c.w[1] << 32);
@@ -85,33 +90,82 @@ __device__ __forceinline__ void dequant_cell(const Cell<BITS, SPARSE>& c, h16x8 
     }
 #pragma unroll
     for (int t = 0; t < 32; ++t) {
-        h16 w = dequant_code<BITS>(codes[t], c.sc, c.ze);
+        h16 w = dequant_code<BITS>(codes[t], sc, ze);
         if (SPARSE && !((c.m >> t) & 1u)) w = (h16)0.0f;
         out[t >> 3][t & 7] = w;
     }
 }
 
+// Fast linear-mode decode of one dense int4 word into 8 fp16 weights in natural
+// k order, bit-exact: the word's low (high) two bytes are replicated into both
+// halves of a register, so that mask-and-OR yields the half2 {1024 + q_even,
+// 64 + q_odd}; subtracting {1024, 64} is exact, then the reference's own two
+// roundings follow: fp16(q - z), fp16(. * s).
+__device__ __forceinline__ h16x8 dequant_word_int4(uint32_t u, h16x2 negz, h16x2 s2) {
+    const uint32_t MSK = 0x00F0000Fu, MAGIC = 0x54006400u;
+    const h16x2 unmagic = {(h16)-1024.0f, (h16)-64.0f};
+    const uint32_t lo = __builtin_amdgcn_perm(u, u, 0x01000100u);    // bytes B0 B1 B0 B1
+    const uint32_t hi = __builtin_amdgcn_perm(u, u, 0x03020302u);    // bytes B2 B3 B2 B3
+    const uint32_t h[4] = {(lo & MSK) | MAGIC, ((lo >> 8) & MSK) | MAGIC,
+                           (hi & MSK) | MAGIC, ((hi >> 8) & MSK) | MAGIC};
+    u32x4 r;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        h16x2 q = as_h2(h[i]) + unmagic;       // exact: {q_even, q_odd}
+        h16x2 d = q + negz;                    // fp16 subtract, one rounding
+        r[i] = as_u32(d * s2);                 // fp16 multiply, one rounding
+    }
+    return bitcast<h16x8>(r);
+}
+
+template <int BITS, bool SPARSE>
+__device__ __forceinline__ void dequant_cell(const Cell<BITS, SPARSE>& c, h16 sc, h16 ze, h16x8 out[4]) {
+    if constexpr (BITS == 4 && !SPARSE) {
+        if (sc >= (h16)0.0f) {
+            const h16x2 negz = {-ze, -ze}, s2 = {sc, sc};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) out[i] = dequant_word_int4(c.w[i], negz, s2);
+            return;
+        }
+    }
+    dequant_cell_generic<BITS, SPARSE>(c, sc, ze, out);
+}
+
+// T threads; thread t owns column t % BN of the weight tile and CPT of its
+// (2 * BN / T) 32-row cells per K step.
 template <int BITS, bool SPARSE, int BM, int BN, int WM, int WN>
-__global__ __launch_bounds__(2 * BN) void matmul_kernel(MatmulArgs a) {
-    constexpr int T = 2 * BN;                     // threads: two per tile column
+__global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 2) void matmul_kernel(MatmulArgs a) {
     constexpr int WAVES_N = BN / WN, WAVES_M = BM / WM;
-    static_assert(WAVES_M * WAVES_N * 64 == T, "wave grid must match the thread count");
+    constexpr int T = WAVES_M * WAVES_N * 64;
     constexpr int TM = WM / 32, TN = WN / 32;     // MFMA tiles per wave
     constexpr int A_CHUNKS = BM * 8 / T;          // 16-byte chunks of the states tile per thread
-    static_assert(BM * 8 % T == 0, "states tile must divide among the threads");
+    constexpr int CPT = 2 * BN / T;               // weight cells per thread
+    static_assert(BM * 8 % T == 0 && (T == BN || T == 2 * BN), "tile/thread mismatch");
+    static_assert(CPT == 1 || CPT == 2, "one or two cells per thread");
 
     __shared__ __attribute__((aligned(16))) h16 As[BM * BK];
     __shared__ __attribute__((aligned(16))) h16 Bs[BK * BN];
 
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const int wm0 = (wave / WAVES_N) * WM, wn0 = (wave % WAVES_N) * WN;
-    const int m0 = blockIdx.y * BM, s0 = blockIdx.x * BN;
+
+    // XCD-aware renumbering: workgroup i runs on XCD i % 8; give each XCD a
+    // contiguous range of column tiles and walk the row tiles fastest.
+    int bid = blockIdx.x;
+    const int total = a.tiles_m * a.tiles_n;
+    {
+        const int per_xcd = (total + 7) / 8;
+        const int xcd = bid % 8, local = bid / 8;
+        const int renum = xcd * per_xcd + local;
+        if (total % 8 == 0) bid = renum;
+    }
+    const int tile_m = bid % a.tiles_m, tile_n = bid / a.tiles_m;
+    const int m0 = tile_m * BM, s0 = tile_n * BN;
     const int64_t boff = blockIdx.z;
     const h16* x = a.x + boff * a.M * (int64_t)a.K;
     h16* outs = a.outs + boff * a.M * (int64_t)a.S;
 
-    // B loader: column n, 32-row block hb of the K step
-    const int bn = t % BN, bhb = t / BN;
+    const int bn = t % BN, bhb0 = (t / BN) * CPT;
     const int bcol = min(s0 + bn, a.S - 1);
 
     f32x16 acc[TM][TN];
@@ -123,7 +177,8 @@ __global__ __launch_bounds__(2 * BN) void matmul_kernel(MatmulArgs a) {
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
     u32x4 areg[A_CHUNKS];
-    Cell<BITS, SPARSE> cell;
+    Cell<BITS, SPARSE> cell[CPT];
+    h16 sc, ze;
 
     auto load_tile = [&](int kt) {
 #pragma unroll
@@ -132,7 +187,11 @@ __global__ __launch_bounds__(2 * BN) void matmul_kernel(MatmulArgs a) {
             const int row = min(m0 + m, a.M - 1);
             areg[i] = *reinterpret_cast<const u32x4*>(x + (int64_t)row * a.K + kt * BK + kc * 8);
         }
-        load_cell<BITS, SPARSE>(cell, a, kt * 2 + bhb, bcol);
+#pragma unroll
+        for (int q = 0; q < CPT; ++q) load_cell<BITS, SPARSE>(cell[q], a, kt * 2 + bhb0 + q, bcol);
+        const int64_t gofs = (int64_t)(kt / a.group_units) * a.S + bcol;
+        sc = a.scales[gofs];
+        ze = a.zeros[gofs];
     };
 
     const int ktiles = a.K / BK;
@@ -144,12 +203,13 @@ __global__ __launch_bounds__(2 * BN) void matmul_kernel(MatmulArgs a) {
             const int c = t + T * i, m = c >> 3, kc = c & 7;
             *reinterpret_cast<u32x4*>(&As[m * BK + ((kc ^ a_swz(m)) << 3)]) = areg[i];
         }
-        {
-            h16x8 w[4];
-            dequant_cell<BITS, SPARSE>(cell, w);
 #pragma unroll
-            for (int q = 0; q < 4; ++q)
-                *reinterpret_cast<h16x8*>(&Bs[((bhb * 4 + q) * BN + bn) * 8]) = w[q];
+        for (int q = 0; q < CPT; ++q) {
+            h16x8 w[4];
+            dequant_cell<BITS, SPARSE>(cell[q], sc, ze, w);
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                *reinterpret_cast<h16x8*>(&Bs[(((bhb0 + q) * 4 + e) * BN + bn) * 8]) = w[e];
         }
         __syncthreads();
         if (kt + 1 < ktiles) load_tile(kt + 1);
@@ -192,11 +252,236 @@ __global__ __launch_bounds__(2 * BN) void matmul_kernel(MatmulArgs a) {
         }
 }
 
+// ---- pipelined variant for dense int4, 256 x 256 tile, 8 waves of 128 x 64.
+// LDS holds two stages of both operand tiles (128 KB, one barrier per K step):
+//  * states go global -> LDS directly (global_load_lds, 16 bytes per lane, no
+//    registers), one K step ahead; the XOR swizzle is applied on the global
+//    side because lane l of such a load always lands at LDS base + 16 l;
+//  * packed weights go global -> registers two K steps ahead, and are decoded
+//    and stored to the other B stage one word at a time between the MFMAs of
+//    the current step, so VALU, LDS and the matrix core overlap inside a wave;
+//  * MFMA operand fragments are fetched one 16-wide k slice ahead.
+// The steady-state loop body has no branches (the last two K steps and
+// exponent-mode groups run separately compiled bodies).
+typedef const __attribute__((address_space(1))) void* gptr_t;
+typedef __attribute__((address_space(3))) void* lptr_t;
+
+__global__ __launch_bounds__(512) void matmul_kernel_pipe(MatmulArgs a) {
+    constexpr int BM = 256, BN = 256, WM = 128, WN = 64, T = 512, TM = 4, TN = 2;
+    constexpr int A_STAGE = BM * BK, B_STAGE = BK * BN;            // halves per stage
+
+    extern __shared__ __attribute__((aligned(16))) char smem_raw[];
+    h16* As0 = reinterpret_cast<h16*>(smem_raw);
+    h16* Bs0 = As0 + 2 * A_STAGE;
+
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int wm0 = (wave >> 2) * WM, wn0 = (wave & 3) * WN;
+
+    int bid = blockIdx.x;
+    const int total = a.tiles_m * a.tiles_n;
+    if (total % 8 == 0) bid = (bid % 8) * (total / 8) + bid / 8;     // XCD-aware renumbering
+    const int tile_m = bid % a.tiles_m, tile_n = bid / a.tiles_m;
+    const int m0 = tile_m * BM, s0 = tile_n * BN;
+    const int64_t boff = blockIdx.z;
+    const h16* x = a.x + boff * a.M * (int64_t)a.K;
+    h16* outs = a.outs + boff * a.M * (int64_t)a.S;
+
+    // states: instruction i of this wave fills rows (8 i + wave) * 8 .. + 8 of the stage.
+    // The tile is required to lie inside the matrix (the launcher guarantees it),
+    // so the four source rows of a lane are 64 rows apart: one offset register.
+    const h16* a_src;
+    {
+        const int m = wave * 8 + (lane >> 3);
+        const int kc = (lane & 7) ^ a_swz(m);          // a_swz(m + 64 i) == a_swz(m)
+        a_src = x + (int64_t)(m0 + m) * a.K + kc * 8;
+    }
+    const int64_t a_row64 = (int64_t)64 * a.K;
+    auto load_a = [&](int kt, int buf) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            __builtin_amdgcn_global_load_lds((gptr_t)(a_src + i * a_row64 + kt * BK),
+                                             (lptr_t)(As0 + buf * A_STAGE + (i * 8 + wave) * 512), 16, 0, 0);
+    };
+
+    // weights: thread owns column bn, 32-row block bhb of every K step
+    const int bn = t & 255, bhb = t >> 8;
+    const int bcol = s0 + bn;
+    struct Stage { uint32_t w[4]; h16 sc, ze; };
+    Stage st[2];
+    auto load_b = [&](Stage& s, int kt) {
+        const uint32_t* p = a.matrix + (int64_t)(kt * 2 + bhb) * 4 * a.S + bcol;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) s.w[r] = p[(int64_t)r * a.S];
+        const int64_t gofs = (int64_t)(kt / a.group_units) * a.S + bcol;
+        s.sc = a.scales[gofs];
+        s.ze = a.zeros[gofs];
+    };
+    auto write_b_fast = [&](const Stage& s, int buf, int q) {
+        const h16x2 negz = {-s.ze, -s.ze}, s2 = {s.sc, s.sc};
+        *reinterpret_cast<h16x8*>(&Bs0[buf * B_STAGE + ((bhb * 4 + q) * BN + bn) * 8]) =
+            dequant_word_int4(s.w[q], negz, s2);
+    };
+    auto write_b_general = [&](const Stage& s, int buf) {
+        Cell<4, false> c;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) c.w[r] = s.w[r];
+        c.m = 0xFFFFFFFFu;
+        h16x8 w[4];
+        dequant_cell_generic<4, false>(c, s.sc, s.ze, w);
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            *reinterpret_cast<h16x8*>(&Bs0[buf * B_STAGE + ((bhb * 4 + e) * BN + bn) * 8]) = w[e];
+    };
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    // fragment addresses (halves, inside a stage) for k slice 0; slice ks adds to kc
+    int a_frag[TM], b_frag[TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i) a_frag[i] = (wm0 + i * 32 + (lane & 31)) * BK;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) b_frag[j] = (wn0 + j * 32 + (lane & 31)) * 8;
+    const int a_sw = a_swz(lane & 31);                // rows differ by multiples of 32: same swizzle
+    auto load_frags = [&](int buf, int ks, h16x8 fa[TM], h16x8 fb[TN]) {
+        const int kc = 2 * ks + (lane >> 5);
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+            fa[i] = *reinterpret_cast<const h16x8*>(&As0[buf * A_STAGE + a_frag[i] + ((kc ^ a_sw) << 3)]);
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+            fb[j] = *reinterpret_cast<const h16x8*>(&Bs0[buf * B_STAGE + kc * BN * 8 + b_frag[j]]);
+    };
+
+    using True = std::integral_constant<bool, true>;
+    using False = std::integral_constant<bool, false>;
+    const int ktiles = a.K / BK;
+
+    // Does any (group, column) of this tile use exponent quantisation (scale < 0
+    // or NaN)?  One pass over the tile's scales (a few KB); the answer is
+    // workgroup-uniform and selects between the pipelined loop, whose decode is
+    // the branch-free linear one, and a plain loop with the general decode.
+    __shared__ int any_expo;
+    if (t == 0) any_expo = 0;
+    __syncthreads();
+    {
+        bool bad = false;
+        const int groups = (ktiles + a.group_units - 1) / a.group_units;
+        for (int g = bhb; g < groups; g += 2) bad |= !(a.scales[(int64_t)g * a.S + bcol] >= (h16)0.0f);
+        if (__builtin_amdgcn_ballot_w64(bad) != 0 && lane == 0) any_expo = 1;
+    }
+    __syncthreads();
+
+    if (any_expo == 0) {
+        // One K step: MFMAs on stage `buf`; meanwhile stage buf^1 is filled for the
+        // next step.  A single branch-free body serves every step: near the end
+        // the loads are clamped to the last K step and their results are unused.
+        const int last = ktiles - 1;
+        auto body = [&](int kt, Stage& cur, Stage& nxt, int buf) {
+            load_a(min(kt + 1, last), buf ^ 1);
+            load_b(cur, min(kt + 2, last));
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks) {
+                h16x8 fa[TM], fb[TN];
+                load_frags(buf, ks, fa, fb);
+                write_b_fast(nxt, buf ^ 1, ks);
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+#pragma unroll
+                    for (int j = 0; j < TN; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+            }
+            __syncthreads();      // also waits for this wave's direct-to-LDS loads and LDS writes
+        };
+        load_a(0, 0);
+        load_b(st[0], 0);
+        load_b(st[1], min(1, last));
+#pragma unroll
+        for (int q = 0; q < 4; ++q) write_b_fast(st[0], 0, q);
+        __syncthreads();
+        int kt = 0;
+        for (; kt + 1 < ktiles; kt += 2) {
+            body(kt, st[0], st[1], 0);
+            body(kt + 1, st[1], st[0], 1);
+        }
+        if (kt < ktiles) body(kt, st[0], st[1], 0);
+    } else {
+        for (int kt = 0; kt < ktiles; ++kt) {
+            load_a(kt, 0);
+            load_b(st[0], kt);
+            write_b_general(st[0], 0);
+            __syncthreads();
+#pragma unroll 1
+            for (int ks = 0; ks < 4; ++ks) {
+                h16x8 fa[TM], fb[TN];
+                load_frags(0, ks, fa, fb);
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+#pragma unroll
+                    for (int j = 0; j < TN; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+            }
+            __syncthreads();
+        }
+    }
+
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const int col = s0 + wn0 + j * 32 + (lane & 31);
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int row = m0 + wm0 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                if (row < a.M && col < a.S) outs[(int64_t)row * a.S + col] = (h16)acc[i][j][r];
+            }
+        }
+}
+
+static void launch_pipe(MatmulArgs a, int64_t B, hipStream_t st) {
+    a.tiles_m = (a.M + 255) / 256;
+    a.tiles_n = (a.S + 255) / 256;
+    const dim3 grid(a.tiles_m * a.tiles_n, 1, (unsigned)B), block(512);
+    constexpr size_t lds = 2 * (size_t)(256 + 256) * BK * sizeof(h16);
+    static bool attr_set = false;       // the attribute sticks to the function for the whole process
+    if (!attr_set) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(matmul_kernel_pipe),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        attr_set = true;
+    }
+    hipLaunchKernelGGL(matmul_kernel_pipe, grid, block, lds, st, a);
+}
+
+template <int BITS, bool SPARSE, int BM, int BN, int WM, int WN>
+static void launch_tile(MatmulArgs a, int64_t B, hipStream_t st) {
+    a.tiles_m = (a.M + BM - 1) / BM;
+    a.tiles_n = (a.S + BN - 1) / BN;
+    const dim3 grid(a.tiles_m * a.tiles_n, 1, (unsigned)B), block((BM / WM) * (BN / WN) * 64);
+    hipLaunchKernelGGL((matmul_kernel<BITS, SPARSE, BM, BN, WM, WN>), grid, block, 0, st, a);
+}
+
 template <int BITS, bool SPARSE>
 static void launch(const MatmulArgs& a, int64_t B, hipStream_t st) {
-    constexpr int BM = 128, BN = 128;
-    const dim3 grid((a.S + BN - 1) / BN, (a.M + BM - 1) / BM, (unsigned)B), block(2 * BN);
-    hipLaunchKernelGGL((matmul_kernel<BITS, SPARSE, BM, BN, 64, 64>), grid, block, 0, st, a);
+    // variant 0 = automatic: the pipelined 256 x 256 kernel where it applies
+    // (dense int4, tile-aligned M and S), otherwise 128 x 256 tiles, and
+    // 128 x 128 tiles for narrow outputs or few rows
+    int variant = (int)tuning(TUNE_MM_VARIANT);
+    const bool pipe_ok = BITS == 4 && !SPARSE && a.M % 256 == 0 && a.S % 256 == 0;
+    if (variant == 5 && !pipe_ok) variant = 0;
+    if (variant == 0) {
+        if (pipe_ok) variant = 5;
+        else if (a.M > 128 && a.S >= 256) variant = 3;
+        else variant = 1;
+    }
+    if (variant == 1) launch_tile<BITS, SPARSE, 128, 128, 64, 64>(a, B, st);
+    else if (variant == 2) launch_tile<BITS, SPARSE, 128, 256, 64, 128>(a, B, st);
+    else if (variant == 3) launch_tile<BITS, SPARSE, 128, 256, 128, 64>(a, B, st);
+    else if (variant == 4) launch_tile<BITS, SPARSE, 256, 256, 128, 64>(a, B, st);
+    else if constexpr (BITS == 4 && !SPARSE) launch_pipe(a, B, st);
 }
 
 }  // namespace i4
@@ -212,7 +497,7 @@ extern "C" int int4mm_matmul(int bits, void* outs, const void* matrix, const voi
     if (rc != INT4MM_OK) return rc;
     const int64_t B = shape->batch, M = shape->seq_len, K = shape->in_size, S = shape->out_size;
     if (B * M * S == 0) return INT4MM_OK;
-    if ((M + 127) / 128 > 65535) return INT4MM_ERR_SHAPE;
+    if (((M + 127) / 128) * ((S + 127) / 128) > 0x7FFFFFFF / 2) return INT4MM_ERR_SHAPE;
     const int64_t g = shape->group_size < 0 ? ONE_GROUP : shape->group_size;
 
     MatmulArgs a;
@@ -226,6 +511,7 @@ extern "C" int int4mm_matmul(int bits, void* outs, const void* matrix, const voi
     a.K = (int)K;
     a.S = (int)S;
     a.group_units = (int)(g / 64 > 0x7FFFFFF ? 0x7FFFFFF : g / 64);
+    a.tiles_m = a.tiles_n = 0;
 
     hipStream_t st = (hipStream_t)stream;
     if (sparse_mask) launch<4, true>(a, B, st);

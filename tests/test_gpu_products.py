@@ -155,3 +155,48 @@ def test_single_group_accepts_1d_scales(H):
         got = outs.cpu().numpy()
         for m in range(M):
             H.assert_product_close(got[:, m:m + 1], exact, f32, kind="vec" if M == 1 else "mtx")
+
+
+# ------------------------------------------------- full-size BASELINE shapes
+def test_full_size_matvec_and_matmul_c2_c3(H):
+    """K=5120, S=20480, g=128 (BASELINE configs 2 and 3): the matvec against the
+    oracle on every output; the M=2048 matmul on 24 sampled rows against the
+    oracle, plus row-linearity of the whole product (a size-independent
+    property: the product of a sum of two row blocks equals the sum of products
+    within fp16 rounding)."""
+    K, S, g = 5120, 20480, 128
+    p = O.make_problem(K=K, S=S, M=1, bits=4, group_size=g, seed=0)
+    d = H.dev_problem(p)
+    exact, f32 = H.oracles(p)
+    got = H.run_capi(p, d, "vec")
+    H.assert_product_close(got, exact, f32)
+    # exponent mode in some columns takes the kernels' general loops at full size
+    M = 2048
+    rng = np.random.default_rng(5)
+    xs = rng.standard_normal((1, M, K), dtype=np.float32).astype(np.float16)
+    pm = dict(p, M=M, states=xs)
+    dm = H.dev_problem(pm)
+    out = H.run_capi(pm, dm, "mtx")
+    rows = np.linspace(0, M - 1, 24).astype(int)
+    w16 = O.dequantize_matrix(4, p["matrix"], p["scales"], p["zeros"], g)
+    want = O.matmul_exact(xs[0, rows], w16)
+    assert O.max_rel_error(want, out[0, rows]) < H.TOL_EXACT_MTX
+    w32 = O.dequantize_matrix_fp32(4, p["matrix"], p["scales"], p["zeros"], g)
+    assert O.max_rel_error(O.matmul_fp32(xs[0, rows], w32), out[0, rows]) < H.TOL_F32
+    # M = 1 through the matmul kernel agrees with the matvec kernel
+    one = H.run_capi(p, d, "mtx")
+    assert O.max_rel_error(got.astype(np.float64), one) < H.TOL_EXACT
+
+
+@pytest.mark.parametrize("M", [256, 512])
+def test_pipelined_matmul_with_exponent_groups(H, M):
+    """tile-aligned dense int4 shapes take the pipelined kernel; negative scales
+    in a few columns force its general loop for the tiles that contain them"""
+    p = O.make_problem(K=512, S=512, M=M, bits=4, group_size=128, seed=21)
+    d = H.dev_problem(p)
+    exact, f32 = H.oracles(p)
+    H.assert_product_close(H.run_capi(p, d, "mtx"), exact, f32, kind="mtx")
+    p["scales"][1, 300:310] *= np.float16(-1)
+    d = H.dev_problem(p)
+    exact, f32 = H.oracles(p)
+    H.assert_product_close(H.run_capi(p, d, "mtx"), exact, f32, kind="mtx")
