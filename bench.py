@@ -28,8 +28,8 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
 MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 MFMA
 
 # HBM bytes per matvec launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see
-# profiles/); None until measured
-MATVEC_TRAFFIC_BYTES = None
+# profiles/matvec_int4_K5120_S20480.md)
+MATVEC_TRAFFIC_BYTES = 57_508_864  # (27580.5 KiB x 2.000 + 1000.0 KiB x 1.000) x 1024
 
 
 def matvec_bytes(K, S, g, bits=4):
@@ -43,6 +43,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-gemm", action="store_true", help="skip the M=2048 matmul leg")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a 256 MiB device-to-device copy five times (a kernel of known HBM "
+                         "traffic, used to scale rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (the matvec/matmul shard "
@@ -131,6 +134,14 @@ def main():
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MATVEC_TRAFFIC_BYTES,
                      "kernel": "i4::matvec_kernel<4,false,...>", "avg_launch_us": round(ev_us, 3)},
     }
+
+    if args.calibrate_copy:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_(0, 255)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        result["calibration"] = {"kernel": "torch device copy", "bytes_read": 256 << 20, "bytes_written": 256 << 20}
 
     # ---- the matmul half of the metric: M=2048, same weights (BASELINE config 3)
     if not args.no_gemm:
