@@ -35,7 +35,7 @@ namespace i4 {
 
 constexpr int MV_MAX_WAVES = 8;
 constexpr int MV_MAX_SPLITS = 32;          // slots per column in the workspace
-constexpr int MV_MAX_UNITS_WG = 1024;     // LDS staging: 128 B of states + 8 B of sums per unit
+constexpr int MV_MAX_UNITS_WG = 384;      // LDS staging: up to 168 B per unit, 64 KB in all
 
 struct MatvecArgs {
     h16* outs;
@@ -54,10 +54,11 @@ struct MatvecArgs {
 
 // ------------------------------------------------------------------ formats
 template <int BITS, bool SPARSE> struct Fmt;
-template <> struct Fmt<4, false> { static constexpr int ROWS = 8, MROWS = 0; static constexpr bool FAST = true; };
-template <> struct Fmt<3, false> { static constexpr int ROWS = 6, MROWS = 0; static constexpr bool FAST = false; };
-template <> struct Fmt<2, false> { static constexpr int ROWS = 4, MROWS = 0; static constexpr bool FAST = true; };
-template <> struct Fmt<4, true>  { static constexpr int ROWS = 4, MROWS = 2; static constexpr bool FAST = false; };
+// ROWS / MROWS: packed weight / mask rows per unit; XS: bytes of staged states per unit
+template <> struct Fmt<4, false> { static constexpr int ROWS = 8, MROWS = 0, XS = 128; static constexpr bool FAST = true; };
+template <> struct Fmt<3, false> { static constexpr int ROWS = 6, MROWS = 0, XS = 160; static constexpr bool FAST = true; };
+template <> struct Fmt<2, false> { static constexpr int ROWS = 4, MROWS = 0, XS = 128; static constexpr bool FAST = true; };
+template <> struct Fmt<4, true>  { static constexpr int ROWS = 4, MROWS = 2, XS = 128; static constexpr bool FAST = false; };
 
 template <int BITS, bool SPARSE>
 struct Unit {
@@ -165,7 +166,66 @@ __device__ __forceinline__ void unit_fast(const Unit<2, false>& u, const h16* xp
         }
     }
 }
-__device__ __forceinline__ void unit_fast(const Unit<3, false>&, const h16*, f32x4[4]) {}
+
+// int3: every 32 codes of a column are a 96-bit stream over three words, code j
+// at stream bit 3j.  A 32-bit window of the stream that starts at bit 3c-1 has
+// codes c, c+1, c+2 at offsets 1, 4, 7 of its low half and codes c+5, c+6, c+7
+// at offsets 0, 3, 6 of its high half: three mask-and-OR operations turn it into
+// three half2 pairs.  Windows at c = 0, 8, 16, 24 (one shift or funnel shift
+// each) cover 24 codes; the pairs (4,11), (12,19), (20,27) come from windows at
+// bits 12, 36, 60 (offsets 0 and 5), codes 3 and 28 from plain shifts.  The
+// states are staged in exactly this pair order, so 26 VALU operations and 9
+// MFMAs process 32 weights.  I3_LO/I3_HI list the code index in the low / high
+// half of pair p (-1: unused, its state is staged as zero); I3_OFF is the magic
+// offset 2^e each code is read with.
+__device__ constexpr int I3_LO[18] = {0, 1, 2, 8, 9, 10, 16, 17, 18, 24, 25, 26, 4, 12, 20, 3, 28, -1};
+__device__ constexpr int I3_HI[18] = {5, 6, 7, 13, 14, 15, 21, 22, 23, 29, 30, 31, 11, 19, 27, -1, -1, -1};
+__device__ constexpr float I3_OFF[32] = {512, 64, 8, 1024, 1024, 1024, 128, 16, 512, 64, 8, 32, 1024, 1024, 128, 16,
+                                         512, 64, 8, 32, 1024, 1024, 128, 16, 512, 64, 8, 32, 1024, 1024, 128, 16};
+
+__device__ __forceinline__ void unit_fast(const Unit<3, false>& u, const h16* xp, f32x4 acc[4]) {
+    const uint32_t MA1 = in_vgpr(0x0007000Eu), GA1 = in_vgpr(0x64006000u);   // {512 + c, 1024 + c5}
+    const uint32_t MA2 = in_vgpr(0x00380070u), GA2 = in_vgpr(0x58005400u);   // {64 + c1, 128 + c6}
+    const uint32_t MA3 = in_vgpr(0x01C00380u), GA3 = in_vgpr(0x4C004800u);   // {8 + c2, 16 + c7}
+    const uint32_t ML = in_vgpr(0x00E00007u), GL = in_vgpr(0x50006400u);     // {1024 + lo, 32 + hi}
+    const uint32_t MS = in_vgpr(0x00000007u), GS = in_vgpr(0x64006400u);     // {1024 + lo, 1024}
+#pragma unroll
+    for (int hb = 0; hb < 2; ++hb) {
+        const uint32_t* xw = reinterpret_cast<const uint32_t*>(xp) + hb * 20;
+        const u32x4 p0 = *reinterpret_cast<const u32x4*>(xw), p1 = *reinterpret_cast<const u32x4*>(xw + 4),
+                    p2 = *reinterpret_cast<const u32x4*>(xw + 8), p3 = *reinterpret_cast<const u32x4*>(xw + 12);
+        const u32x2 p4 = *reinterpret_cast<const u32x2*>(xw + 16);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const uint32_t w0 = u.w[3 * hb][c], w1 = u.w[3 * hb + 1][c], w2 = u.w[3 * hb + 2][c];
+            const uint32_t a0 = w0 << 1, a1 = __builtin_amdgcn_alignbit(w1, w0, 23),
+                           a2 = __builtin_amdgcn_alignbit(w2, w1, 15), a3 = w2 >> 7;
+            const uint32_t l0 = __builtin_amdgcn_alignbit(w1, w0, 12), l1 = __builtin_amdgcn_alignbit(w2, w1, 4),
+                           l2 = __builtin_amdgcn_alignbit(w2, w1, 28);
+            const uint32_t s3 = w0 >> 9, s28 = w2 >> 20;
+            f32x4 r = acc[c];
+            r = mma4(p0.x, p0.y, and_or(a0, MA1, GA1), and_or(a0, MA2, GA2), r);
+            r = mma4(p0.z, p0.w, and_or(a0, MA3, GA3), and_or(a1, MA1, GA1), r);
+            r = mma4(p1.x, p1.y, and_or(a1, MA2, GA2), and_or(a1, MA3, GA3), r);
+            r = mma4(p1.z, p1.w, and_or(a2, MA1, GA1), and_or(a2, MA2, GA2), r);
+            r = mma4(p2.x, p2.y, and_or(a2, MA3, GA3), and_or(a3, MA1, GA1), r);
+            r = mma4(p2.z, p2.w, and_or(a3, MA2, GA2), and_or(a3, MA3, GA3), r);
+            r = mma4(p3.x, p3.y, and_or(l0, ML, GL), and_or(l1, ML, GL), r);
+            r = mma4(p3.z, p3.w, and_or(l2, ML, GL), and_or(s3, MS, GS), r);
+            const uint32_t last = and_or(s28, MS, GS);
+            r = mma4(p4.x, p4.y, last, last, r);          // second pair is unused: its states are zero
+            acc[c] = r;
+        }
+    }
+}
+
+// byte selector of v_perm_b32(hi_src, lo_src, sel) that builds the half2 {state a, state b}
+// from the natural-order dwords holding them; -1 selects zero
+__host__ __device__ constexpr uint32_t pair_selector(int a, int b) {
+    const uint32_t lo = a < 0 ? 0x0C0Cu : (uint32_t)(((a & 1) * 2 + 1) << 8 | ((a & 1) * 2));
+    const uint32_t hi = b < 0 ? 0x0C0Cu : (uint32_t)((4 + (b & 1) * 2 + 1) << 8 | (4 + (b & 1) * 2));
+    return hi << 16 | lo;
+}
 __device__ __forceinline__ void unit_fast(const Unit<4, true>&, const h16*, f32x4[4]) {}
 
 template <int BITS>
@@ -267,7 +327,7 @@ void matvec_kernel(MatvecArgs a) {
     // same memory is reused for the final reduction
     extern __shared__ __attribute__((aligned(16))) char smem[];
     h16* xs = reinterpret_cast<h16*>(smem);
-    float* sums = reinterpret_cast<float*>(smem + (size_t)a.units_per_wg * 128);
+    float* sums = reinterpret_cast<float*>(smem + (size_t)a.units_per_wg * Fmt<BITS, SPARSE>::XS);
     float* red = reinterpret_cast<float*>(smem);
 
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6, nwaves = blockDim.x >> 6;
@@ -283,16 +343,21 @@ void matvec_kernel(MatvecArgs a) {
     // ---- issue order matters: loads return in order, so the (small) loads of
     // the states go first and the weight loads follow; the staging below then
     // only waits for the states while the weights are still in flight.
-    constexpr int HPR = BITS == 2 ? 16 : 8;       // halves (k values) per staged row
-    constexpr int RPU = 64 / HPR;                 // staged rows per unit
-    const int nrows = FAST ? (wg_u1 - wg_u0) * RPU : 0;
-    const int nrows8 = (nrows + 7) & ~7;
+    // A staging item is what one thread permutes: one packed row's worth of
+    // states for int4 / int2 (8 / 16 halves), one 32-row cell for int3.
+    constexpr int ITEM_H = BITS == 4 ? 8 : (BITS == 2 ? 16 : 32);   // halves per item
+    constexpr int IPU = 64 / ITEM_H;                                  // items per unit
+    constexpr int ITEM_V = ITEM_H / 8;                                // 16-byte loads per item
+    const int nitems = FAST ? (wg_u1 - wg_u0) * IPU : 0;
+    const int nitems8 = (nitems + 7) & ~7;
     const h16* xg = a.x + wg_u0 * 64;
-    u32x4 xa = {0, 0, 0, 0}, xb = {0, 0, 0, 0};
+    u32x4 xv[ITEM_V];
+#pragma unroll
+    for (int i = 0; i < ITEM_V; ++i) xv[i] = u32x4{0, 0, 0, 0};
     auto load_x = [&](int r) {
-        if (r < nrows) {
-            xa = *reinterpret_cast<const u32x4*>(xg + r * HPR);
-            if constexpr (HPR == 16) xb = *reinterpret_cast<const u32x4*>(xg + r * HPR + 8);
+        if (r < nitems) {
+#pragma unroll
+            for (int i = 0; i < ITEM_V; ++i) xv[i] = *reinterpret_cast<const u32x4*>(xg + r * ITEM_H + i * 8);
         }
     };
     if constexpr (FAST) load_x(t);
@@ -307,12 +372,12 @@ void matvec_kernel(MatvecArgs a) {
     }
 
     if constexpr (FAST) {
-        for (int r = t; r < nrows8; r += blockDim.x) {
+        for (int r = t; r < nitems8; r += blockDim.x) {
             if (r != t) load_x(r);
             float s = 0.f, o = 0.f;
-            if (r < nrows) {
+            if (r < nitems) {
                 if constexpr (BITS == 4) {
-                    const u32x4 v = xa;                                           // x0x1 x2x3 x4x5 x6x7
+                    const u32x4 v = xv[0];                                         // x0x1 x2x3 x4x5 x6x7
                     u32x4 p;
                     p.x = __builtin_amdgcn_perm(v.z, v.x, 0x05040100u);            // {x0, x4}
                     p.y = __builtin_amdgcn_perm(v.z, v.x, 0x07060302u);            // {x1, x5}
@@ -323,8 +388,8 @@ void matvec_kernel(MatvecArgs a) {
                     const float d = hi_f32(v.x) + hi_f32(v.y) + hi_f32(v.z) + hi_f32(v.w);
                     s = e + d;
                     o = 1024.f * e + 64.f * d;
-                } else {
-                    const u32x4 va = xa, vb = xb;
+                } else if constexpr (BITS == 2) {
+                    const u32x4 va = xv[0], vb = xv[1];
                     u32x4 pa, pb;
                     pa.x = __builtin_amdgcn_perm(vb.x, va.x, 0x05040100u);         // {x0, x8}
                     pa.y = __builtin_amdgcn_perm(vb.x, va.x, 0x07060302u);         // {x1, x9}
@@ -343,13 +408,35 @@ void matvec_kernel(MatvecArgs a) {
                         s += lo + hi;
                         o += lo * fast_offset<2>(2 * j) + hi * fast_offset<2>(2 * j + 1);
                     }
+                } else {                                                           // int3: one 32-row cell
+                    uint32_t d[16];                                                // d[j] = {x_2j, x_2j+1}
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) { d[4 * i] = xv[i].x; d[4 * i + 1] = xv[i].y; d[4 * i + 2] = xv[i].z; d[4 * i + 3] = xv[i].w; }
+                    uint32_t q[20];
+#pragma unroll
+                    for (int k = 0; k < 18; ++k) {
+                        const int lo = I3_LO[k], hi = I3_HI[k];
+                        q[k] = __builtin_amdgcn_perm(d[hi < 0 ? 0 : hi / 2], d[lo < 0 ? 0 : lo / 2], pair_selector(lo, hi));
+                    }
+                    q[18] = q[19] = 0u;
+                    uint32_t* dst = reinterpret_cast<uint32_t*>(xs) + r * 20;
+#pragma unroll
+                    for (int k = 0; k < 20; k += 4) *reinterpret_cast<u32x4*>(dst + k) = u32x4{q[k], q[k + 1], q[k + 2], q[k + 3]};
+#pragma unroll
+                    for (int j = 0; j < 16; ++j) {
+                        const float lo = lo_f32(d[j]), hi = hi_f32(d[j]);
+                        s += lo + hi;
+                        o += lo * I3_OFF[2 * j] + hi * I3_OFF[2 * j + 1];
+                    }
                 }
             }
-            if constexpr (RPU == 8) { s = sum8(s); o = sum8(o); }
-            else { s = sum4(s); o = sum4(o); }
-            if ((r % RPU) == 0 && r < nrows) {     // first row of a unit publishes its sums
-                sums[(r / RPU) * 2] = s;
-                sums[(r / RPU) * 2 + 1] = o;
+            // sum the items of a unit (aligned groups of IPU lanes)
+            if constexpr (IPU == 8) { s = sum8(s); o = sum8(o); }
+            else if constexpr (IPU == 4) { s = sum4(s); o = sum4(o); }
+            else { s += dpp_f32<0xB1>(s); o += dpp_f32<0xB1>(o); }
+            if ((r % IPU) == 0 && r < nitems) {    // first item of a unit publishes its sums
+                sums[(r / IPU) * 2] = s;
+                sums[(r / IPU) * 2 + 1] = o;
             }
         }
         __syncthreads();
@@ -367,7 +454,7 @@ void matvec_kernel(MatvecArgs a) {
 #pragma unroll
             for (int c = 0; c < 4; ++c) acc[c] = f32x4{0.f, 0.f, 0.f, 0.f};
             const int lu = unit - wg_u0;
-            unit_fast(un, xs + lu * 64, acc);
+            unit_fast(un, xs + lu * (Fmt<BITS, SPARSE>::XS / 2), acc);
             const float xsum = sums[lu * 2], xoff = sums[lu * 2 + 1];
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
@@ -503,7 +590,9 @@ void matvec_kernel(MatvecArgs a) {
 }
 
 template <int BITS, bool SPARSE>
-static void launch(const MatvecArgs& a, int lk, bool pf, dim3 grid, dim3 block, size_t lds, hipStream_t st) {
+static void launch(const MatvecArgs& a, int lk, bool pf, dim3 grid, dim3 block, hipStream_t st) {
+    size_t lds = (size_t)a.units_per_wg * (Fmt<BITS, SPARSE>::XS + 8);     // staged states + per-unit sums
+    if (lds < (size_t)block.x * 16) lds = (size_t)block.x * 16;           // reduction area: 4 floats per thread
 #define I4_LAUNCH(LK_, PF_) hipLaunchKernelGGL((matvec_kernel<BITS, SPARSE, LK_, PF_>), grid, block, lds, st, a)
     if (lk == 1) { if (pf) I4_LAUNCH(1, true); else I4_LAUNCH(1, false); }
     else if (lk == 2) { if (pf) I4_LAUNCH(2, true); else I4_LAUNCH(2, false); }
@@ -574,17 +663,15 @@ extern "C" int int4mm_matvec(int bits, void* outs, const void* matrix, const voi
     a.group_units = (int)(g / 64 > 0x7FFFFFF ? 0x7FFFFFF : g / 64);
     a.splits = splits;
 
-    size_t lds = (size_t)upwg * 136;
-    if (lds < (size_t)waves * 1024) lds = (size_t)waves * 1024;
     const dim3 grid(strips, splits, 1), block(waves * WAVE);
     hipStream_t st = (hipStream_t)stream;
     for (int64_t b = 0; b < B; ++b) {                      // one pass over the weights per batch row
         a.outs = (h16*)outs + b * S;
         a.x = (const h16*)multiplier + b * K;
-        if (sparse_mask) launch<4, true>(a, lk, pf, grid, block, lds, st);
-        else if (bits == 4) launch<4, false>(a, lk, pf, grid, block, lds, st);
-        else if (bits == 3) launch<3, false>(a, lk, pf, grid, block, lds, st);
-        else launch<2, false>(a, lk, pf, grid, block, lds, st);
+        if (sparse_mask) launch<4, true>(a, lk, pf, grid, block, st);
+        else if (bits == 4) launch<4, false>(a, lk, pf, grid, block, st);
+        else if (bits == 3) launch<3, false>(a, lk, pf, grid, block, st);
+        else launch<2, false>(a, lk, pf, grid, block, st);
         rc = check_launch("matvec");
         if (rc != INT4MM_OK) return rc;
     }
