@@ -35,7 +35,7 @@ namespace i4 {
 
 constexpr int MV_MAX_WAVES = 8;
 constexpr int MV_MAX_SPLITS = 32;          // slots per column in the workspace
-constexpr int MV_MAX_UNITS_WG = 384;      // LDS staging: up to 168 B per unit, 64 KB in all
+constexpr int MV_MAX_UNITS_WG = 224;      // LDS staging: up to 264 B per unit, 64 KB in all
 
 struct MatvecArgs {
     h16* outs;
@@ -58,7 +58,7 @@ template <int BITS, bool SPARSE> struct Fmt;
 template <> struct Fmt<4, false> { static constexpr int ROWS = 8, MROWS = 0, XS = 128; static constexpr bool FAST = true; };
 template <> struct Fmt<3, false> { static constexpr int ROWS = 6, MROWS = 0, XS = 160; static constexpr bool FAST = true; };
 template <> struct Fmt<2, false> { static constexpr int ROWS = 4, MROWS = 0, XS = 128; static constexpr bool FAST = true; };
-template <> struct Fmt<4, true>  { static constexpr int ROWS = 4, MROWS = 2, XS = 128; static constexpr bool FAST = false; };
+template <> struct Fmt<4, true>  { static constexpr int ROWS = 4, MROWS = 2, XS = 256; static constexpr bool FAST = true; };
 
 template <int BITS, bool SPARSE>
 struct Unit {
@@ -226,6 +226,60 @@ __host__ __device__ constexpr uint32_t pair_selector(int a, int b) {
     const uint32_t hi = b < 0 ? 0x0C0Cu : (uint32_t)((4 + (b & 1) * 2 + 1) << 8 | (4 + (b & 1) * 2));
     return hi << 16 | lo;
 }
+
+// 16:32 sparse int4.  Per (32-row block, column): a mask word and 16 kept codes
+// packed in 64 bits.  Two dot products are needed per column: A = sum over kept
+// rows of x*q and M = sum over kept rows of x (dropped rows contribute exactly 0).
+//  * M treats the mask word as 32 one-bit codes: (m >> 4i) & (0x00010001 << o) |
+//    magic gives the half2 {2^(10-o) + bit(4i+o), 2^(10-o) + bit(16+4i+o)}.
+//  * A first expands the kept codes to their rows.  The mask is taken a byte at
+//    a time: the next eight nibbles of the code stream are split into eight
+//    bytes (even / odd nibbles of one word), and a 256-entry table in LDS holds,
+//    for every mask byte, the four v_perm selectors that route the right code
+//    byte (or zero) into the 16-bit halves of the pairs (row j, row j+4) of that
+//    byte's eight rows; OR-ing 0x6400 into both halves makes them 1024 + q.
+// Staged states per unit: for each block 16 dwords {x_j, x_j+4} ordered as the
+// dense int4 path, then for each block 16 dwords {x_p, x_p+16}.
+__device__ __forceinline__ void unit_fast_sparse(const Unit<4, true>& u, const h16* xp, const u32x4* lut,
+                                                 f32x4 accA[4], f32x4 accM[4]) {
+    const uint32_t NIB = in_vgpr(0x0F0F0F0Fu), G10 = in_vgpr(0x64006400u);
+    const uint32_t B0 = in_vgpr(0x00010001u), B1 = in_vgpr(0x00020002u), B2 = in_vgpr(0x00040004u),
+                   B3 = in_vgpr(0x00080008u);
+    const uint32_t G9 = in_vgpr(0x60006000u), G8 = in_vgpr(0x5C005C00u), G7 = in_vgpr(0x58005800u);
+    const uint32_t* xw = reinterpret_cast<const uint32_t*>(xp);
+#pragma unroll
+    for (int hb = 0; hb < 2; ++hb) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const uint32_t m = u.m[hb][c];
+            uint64_t stream = (uint64_t)u.w[2 * hb][c] | ((uint64_t)u.w[2 * hb + 1][c] << 32);
+            f32x4 ra = accA[c], rm = accM[c];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                // ---- rows 8i .. 8i+7: expand and accumulate x*q
+                const uint32_t mb = (m >> (8 * i)) & 0xFFu;
+                const u32x4 sel = lut[mb];
+                const uint32_t chunk = (uint32_t)stream;
+                const uint32_t even = chunk & NIB, odd = (chunk >> 4) & NIB;
+                stream >>= 4 * __builtin_popcount(mb);
+                const u32x4 px = *reinterpret_cast<const u32x4*>(xw + hb * 16 + i * 4);
+                const uint32_t b0 = __builtin_amdgcn_perm(odd, even, sel.x) | G10;
+                const uint32_t b1 = __builtin_amdgcn_perm(odd, even, sel.y) | G10;
+                const uint32_t b2 = __builtin_amdgcn_perm(odd, even, sel.z) | G10;
+                const uint32_t b3 = __builtin_amdgcn_perm(odd, even, sel.w) | G10;
+                ra = mma4(px.x, px.y, b0, b1, ra);
+                ra = mma4(px.z, px.w, b2, b3, ra);
+                // ---- mask bits 4i .. 4i+3 and 16+4i .. 16+4i+3: accumulate x over kept rows
+                const uint32_t ms = m >> (4 * i);
+                const u32x4 pm = *reinterpret_cast<const u32x4*>(xw + 32 + hb * 16 + i * 4);
+                rm = mma4(pm.x, pm.y, and_or(ms, B0, G10), and_or(ms, B1, G9), rm);
+                rm = mma4(pm.z, pm.w, and_or(ms, B2, G8), and_or(ms, B3, G7), rm);
+            }
+            accA[c] = ra;
+            accM[c] = rm;
+        }
+    }
+}
 __device__ __forceinline__ void unit_fast(const Unit<4, true>&, const h16*, f32x4[4]) {}
 
 template <int BITS>
@@ -329,6 +383,9 @@ void matvec_kernel(MatvecArgs a) {
     h16* xs = reinterpret_cast<h16*>(smem);
     float* sums = reinterpret_cast<float*>(smem + (size_t)a.units_per_wg * Fmt<BITS, SPARSE>::XS);
     float* red = reinterpret_cast<float*>(smem);
+    // 16:32 only: table of v_perm selectors per mask byte, behind the sums (the final
+    // reduction reuses the front of the buffer, which never reaches the table)
+    u32x4* lut = reinterpret_cast<u32x4*>(smem + (((size_t)a.units_per_wg * (Fmt<BITS, SPARSE>::XS + 8) + 15) & ~(size_t)15));
 
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6, nwaves = blockDim.x >> 6;
     const int cl = lane % LC, kl = lane / LC;
@@ -344,8 +401,8 @@ void matvec_kernel(MatvecArgs a) {
     // the states go first and the weight loads follow; the staging below then
     // only waits for the states while the weights are still in flight.
     // A staging item is what one thread permutes: one packed row's worth of
-    // states for int4 / int2 (8 / 16 halves), one 32-row cell for int3.
-    constexpr int ITEM_H = BITS == 4 ? 8 : (BITS == 2 ? 16 : 32);   // halves per item
+    // states for int4 / int2 (8 / 16 halves), one 32-row cell for int3 and 16:32.
+    constexpr int ITEM_H = SPARSE ? 32 : (BITS == 4 ? 8 : (BITS == 2 ? 16 : 32));   // halves per item
     constexpr int IPU = 64 / ITEM_H;                                  // items per unit
     constexpr int ITEM_V = ITEM_H / 8;                                // 16-byte loads per item
     const int nitems = FAST ? (wg_u1 - wg_u0) * IPU : 0;
@@ -371,12 +428,61 @@ void matvec_kernel(MatvecArgs a) {
         if (work_b) load_unit(ub, a, u + ng, col);
     }
 
+    if constexpr (SPARSE) {
+        // selector table: for mask byte b, pair j = (row j, row j+4): byte 0 picks the code of
+        // row j from the pool {even nibbles, odd nibbles}, byte 2 that of row j+4; 0x0C yields 0
+        for (int b = t; b < 256; b += blockDim.x) {
+            uint32_t selb[8];
+            int rank = 0;
+#pragma unroll
+            for (int p8 = 0; p8 < 8; ++p8) {
+                const bool k = (b >> p8) & 1;
+                selb[p8] = k ? (uint32_t)((rank & 1) * 4 + (rank >> 1)) : 0x0Cu;
+                rank += k;
+            }
+            u32x4 e;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) e[j] = selb[j] | (0x0Cu << 8) | (selb[j + 4] << 16) | (0x0Cu << 24);
+            lut[b] = e;
+        }
+    }
     if constexpr (FAST) {
         for (int r = t; r < nitems8; r += blockDim.x) {
             if (r != t) load_x(r);
             float s = 0.f, o = 0.f;
             if (r < nitems) {
-                if constexpr (BITS == 4) {
+                if constexpr (SPARSE) {                                            // one 32-row block
+                    uint32_t d[16];                                                // d[j] = {x_2j, x_2j+1}
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) { d[4 * i] = xv[i].x; d[4 * i + 1] = xv[i].y; d[4 * i + 2] = xv[i].z; d[4 * i + 3] = xv[i].w; }
+                    uint32_t* dstA = reinterpret_cast<uint32_t*>(xs) + (r >> 1) * 64 + (r & 1) * 16;
+                    uint32_t* dstM = dstA + 32;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {                                  // rows 8i..8i+7: {x_j, x_j+4}
+                        u32x4 p;
+                        p.x = __builtin_amdgcn_perm(d[4 * i + 2], d[4 * i], 0x05040100u);
+                        p.y = __builtin_amdgcn_perm(d[4 * i + 2], d[4 * i], 0x07060302u);
+                        p.z = __builtin_amdgcn_perm(d[4 * i + 3], d[4 * i + 1], 0x05040100u);
+                        p.w = __builtin_amdgcn_perm(d[4 * i + 3], d[4 * i + 1], 0x07060302u);
+                        *reinterpret_cast<u32x4*>(dstA + 4 * i) = p;
+                    }
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {                                  // {x_p, x_p+16}, p = 4i..4i+3
+                        u32x4 p;
+                        p.x = __builtin_amdgcn_perm(d[8 + 2 * i], d[2 * i], 0x05040100u);
+                        p.y = __builtin_amdgcn_perm(d[8 + 2 * i], d[2 * i], 0x07060302u);
+                        p.z = __builtin_amdgcn_perm(d[9 + 2 * i], d[2 * i + 1], 0x05040100u);
+                        p.w = __builtin_amdgcn_perm(d[9 + 2 * i], d[2 * i + 1], 0x07060302u);
+                        *reinterpret_cast<u32x4*>(dstM + 4 * i) = p;
+                    }
+                    // s: offset of the code part (1024 for every row); o: offset of the mask part
+#pragma unroll
+                    for (int j = 0; j < 16; ++j) {
+                        const float lo = lo_f32(d[j]), hi = hi_f32(d[j]);
+                        s += 1024.f * (lo + hi);
+                        o += lo * (float)(1024 >> ((2 * j) & 3)) + hi * (float)(1024 >> ((2 * j + 1) & 3));
+                    }
+                } else if constexpr (BITS == 4) {
                     const u32x4 v = xv[0];                                         // x0x1 x2x3 x4x5 x6x7
                     u32x4 p;
                     p.x = __builtin_amdgcn_perm(v.z, v.x, 0x05040100u);            // {x0, x4}
@@ -449,7 +555,20 @@ void matvec_kernel(MatvecArgs a) {
         float sc[4], ze[4];
         bool expo[4];
         unpack_params(un.sc, un.ze, sc, ze, expo);
-        if constexpr (FAST) {
+        if constexpr (FAST && SPARSE) {
+            f32x4 accA[4], accM[4];
+#pragma unroll
+            for (int c = 0; c < 4; ++c) { accA[c] = f32x4{0.f, 0.f, 0.f, 0.f}; accM[c] = f32x4{0.f, 0.f, 0.f, 0.f}; }
+            const int lu = unit - wg_u0;
+            unit_fast_sparse(un, xs + lu * (Fmt<BITS, SPARSE>::XS / 2), lut, accA, accM);
+            const float offA = sums[lu * 2], offM = sums[lu * 2 + 1];
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const float sl = fmaxf(sc[c], 0.f);
+                y[c] += sl * ((accA[c][0] - offA) - ze[c] * (accM[c][0] - offM));
+                need_general |= expo[c];
+            }
+        } else if constexpr (FAST) {
             f32x4 acc[4];
 #pragma unroll
             for (int c = 0; c < 4; ++c) acc[c] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -592,6 +711,7 @@ void matvec_kernel(MatvecArgs a) {
 template <int BITS, bool SPARSE>
 static void launch(const MatvecArgs& a, int lk, bool pf, dim3 grid, dim3 block, hipStream_t st) {
     size_t lds = (size_t)a.units_per_wg * (Fmt<BITS, SPARSE>::XS + 8);     // staged states + per-unit sums
+    if (SPARSE) lds = ((lds + 15) & ~(size_t)15) + 256 * 16;               // selector table
     if (lds < (size_t)block.x * 16) lds = (size_t)block.x * 16;           // reduction area: 4 floats per thread
 #define I4_LAUNCH(LK_, PF_) hipLaunchKernelGGL((matvec_kernel<BITS, SPARSE, LK_, PF_>), grid, block, lds, st, a)
     if (lk == 1) { if (pf) I4_LAUNCH(1, true); else I4_LAUNCH(1, false); }
