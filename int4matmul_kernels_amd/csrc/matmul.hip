@@ -252,86 +252,91 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 2) void matmul_kernel(M
         }
 }
 
-// ---- pipelined variant for dense int4, 256 x 256 tile, 8 waves of 128 x 64.
-// LDS holds two stages of both operand tiles (128 KB, one barrier per K step):
-//  * states go global -> LDS directly (global_load_lds, 16 bytes per lane, no
-//    registers), one K step ahead; the XOR swizzle is applied on the global
-//    side because lane l of such a load always lands at LDS base + 16 l;
-//  * packed weights go global -> registers two K steps ahead, and are decoded
-//    and stored to the other B stage one word at a time between the MFMAs of
-//    the current step, so VALU, LDS and the matrix core overlap inside a wave;
-//  * MFMA operand fragments are fetched one 16-wide k slice ahead.
-// The steady-state loop body has no branches (the last two K steps and
-// exponent-mode groups run separately compiled bodies).
-typedef const __attribute__((address_space(1))) void* gptr_t;
-typedef __attribute__((address_space(3))) void* lptr_t;
+// ---- pipelined variant for dense int4: (TM * 64) x 256 tile, 8 waves (2 x 4) of
+// (TM * 32) x 64, K steps of 32, four LDS stages of each operand (128 KB).
+//  * states go global -> registers three steps ahead and are stored to the LDS
+//    stage of step k+2 during step k;
+//  * packed weights go global -> registers four steps ahead and are decoded
+//    into the LDS stage of step k+2 one word at a time between the MFMAs of
+//    step k, so VALU, LDS and the matrix core overlap inside a wave;
+//  * MFMA operand fragments are fetched one 16-wide k slice ahead, ACROSS step
+//    boundaries: everything a step reads was complete one barrier earlier, so
+//    the barrier that closes a step orders buffer reuse only and the MFMA
+//    stream never drains while waves wait for each other.
+// The steady-state loop body has no branches; a tile that contains exponent-mode
+// groups takes a plain loop with the general decode instead.
+constexpr int PK = 32;            // K per step of the pipelined kernel
 
-__global__ __launch_bounds__(512) void matmul_kernel_pipe(MatmulArgs a) {
-    constexpr int BM = 256, BN = 256, WM = 128, WN = 64, T = 512, TM = 4, TN = 2;
-    constexpr int A_STAGE = BM * BK, B_STAGE = BK * BN;            // halves per stage
+__device__ __forceinline__ h16x8 dequant_word_generic4(uint32_t w, h16 sc, h16 ze) {
+    h16x8 r;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) r[e] = dequant_code<4>((w >> (4 * e)) & 15u, sc, ze);
+    return r;
+}
 
-    extern __shared__ __attribute__((aligned(16))) char smem_raw[];
-    h16* As0 = reinterpret_cast<h16*>(smem_raw);
-    h16* Bs0 = As0 + 2 * A_STAGE;
+template <int TM>
+__device__ __forceinline__ void pipe_tile(const MatmulArgs& a, const int m0, const int s0, const h16* x,
+                                          h16* outs, h16* As, h16* Bs) {
+    constexpr int BM = TM * 64, BN = 256, WM = TM * 32, WN = 64, TN = 2;
+    constexpr int A_STAGE = 256 * PK, B_STAGE = PK * BN;           // halves per stage (A sized for TM = 4)
+    constexpr int A_LOADS = TM / 2;                                // direct-to-LDS loads per wave and step
 
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const int wm0 = (wave >> 2) * WM, wn0 = (wave & 3) * WN;
 
-    int bid = blockIdx.x;
-    const int total = a.tiles_m * a.tiles_n;
-    if (total % 8 == 0) bid = (bid % 8) * (total / 8) + bid / 8;     // XCD-aware renumbering
-    const int tile_m = bid % a.tiles_m, tile_n = bid / a.tiles_m;
-    const int m0 = tile_m * BM, s0 = tile_n * BN;
-    const int64_t boff = blockIdx.z;
-    const h16* x = a.x + boff * a.M * (int64_t)a.K;
-    h16* outs = a.outs + boff * a.M * (int64_t)a.S;
-
-    // states: instruction i of this wave fills rows (8 i + wave) * 8 .. + 8 of the stage.
-    // The tile is required to lie inside the matrix (the launcher guarantees it),
-    // so the four source rows of a lane are 64 rows apart: one offset register.
-    const h16* a_src;
-    {
-        const int m = wave * 8 + (lane >> 3);
-        const int kc = (lane & 7) ^ a_swz(m);          // a_swz(m + 64 i) == a_swz(m)
-        a_src = x + (int64_t)(m0 + m) * a.K + kc * 8;
-    }
-    const int64_t a_row64 = (int64_t)64 * a.K;
-    auto load_a = [&](int kt, int buf) {
+    // states stage: row m at m * 64 bytes, 16-byte chunk c of the row stored at
+    // c ^ ((m >> 2) & 3): sixteen consecutive rows read the same logical chunk
+    // from sixteen different bank groups.  Thread t moves chunk t % 4 of rows
+    // t / 4 and t / 4 + 128 through registers.  The tile lies inside the matrix
+    // (launcher's duty).
+    struct AStage { u32x4 v[A_LOADS]; };
+    const int a_row = t >> 2, a_chunk = t & 3;
+    const h16* a_src = x + (int64_t)(m0 + a_row) * a.K + a_chunk * 8;
+    const int64_t a_row128 = (int64_t)128 * a.K;
+    const int a_dst = a_row * PK + ((a_chunk ^ ((a_row >> 2) & 3)) << 3);       // halves; rows + 128: same swizzle
+    auto load_a = [&](AStage& r, int kt) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-            __builtin_amdgcn_global_load_lds((gptr_t)(a_src + i * a_row64 + kt * BK),
-                                             (lptr_t)(As0 + buf * A_STAGE + (i * 8 + wave) * 512), 16, 0, 0);
+        for (int i = 0; i < A_LOADS; ++i)
+            r.v[i] = *reinterpret_cast<const u32x4*>(a_src + i * a_row128 + kt * PK);
+    };
+    auto write_a = [&](const AStage& r, int stage) {
+#pragma unroll
+        for (int i = 0; i < A_LOADS; ++i)
+            *reinterpret_cast<u32x4*>(&As[stage * A_STAGE + i * 128 * PK + a_dst]) = r.v[i];
     };
 
-    // weights: thread owns column bn, 32-row block bhb of every K step
+    // weights: thread owns column bn and packed rows 2 bhb, 2 bhb + 1 of every K step.
+    // scale / zero travel as the aligned 32-bit word that holds the column's half
+    // (sub-dword loads make the compiler wait for every outstanding load); `half_sel`
+    // replicates the wanted half into both lanes of a packed register.
     const int bn = t & 255, bhb = t >> 8;
     const int bcol = s0 + bn;
-    struct Stage { uint32_t w[4]; h16 sc, ze; };
-    Stage st[2];
-    auto load_b = [&](Stage& s, int kt) {
-        const uint32_t* p = a.matrix + (int64_t)(kt * 2 + bhb) * 4 * a.S + bcol;
-#pragma unroll
-        for (int r = 0; r < 4; ++r) s.w[r] = p[(int64_t)r * a.S];
-        const int64_t gofs = (int64_t)(kt / a.group_units) * a.S + bcol;
-        s.sc = a.scales[gofs];
-        s.ze = a.zeros[gofs];
+    struct Stage { uint32_t w[2]; uint32_t sc, ze; };
+    const uint32_t half_sel = (bcol & 1) ? 0x03020302u : 0x01000100u;
+    const uint32_t* b_base = a.matrix + (int64_t)bhb * 2 * a.S + bcol;
+    const int64_t b_step = (int64_t)4 * a.S;
+    const h16* sc_base = a.scales + (bcol & ~1);
+    const h16* ze_base = a.zeros + (bcol & ~1);
+    auto load_b = [&](Stage& s, int kt, int group) {
+        const uint32_t* p = b_base + kt * b_step;
+        s.w[0] = p[0];
+        s.w[1] = p[a.S];
+        s.sc = *reinterpret_cast<const uint32_t*>(sc_base + (int64_t)group * a.S);
+        s.ze = *reinterpret_cast<const uint32_t*>(ze_base + (int64_t)group * a.S);
     };
-    auto write_b_fast = [&](const Stage& s, int buf, int q) {
-        const h16x2 negz = {-s.ze, -s.ze}, s2 = {s.sc, s.sc};
-        *reinterpret_cast<h16x8*>(&Bs0[buf * B_STAGE + ((bhb * 4 + q) * BN + bn) * 8]) =
-            dequant_word_int4(s.w[q], negz, s2);
+    auto stage_scale = [&](const Stage& s) { return as_h2(__builtin_amdgcn_perm(s.sc, s.sc, half_sel)); };
+    auto stage_negzero = [&](const Stage& s) {
+        return as_h2(__builtin_amdgcn_perm(s.ze, s.ze, half_sel) ^ 0x80008000u);
     };
-    auto write_b_general = [&](const Stage& s, int buf) {
-        Cell<4, false> c;
-#pragma unroll
-        for (int r = 0; r < 4; ++r) c.w[r] = s.w[r];
-        c.m = 0xFFFFFFFFu;
-        h16x8 w[4];
-        dequant_cell_generic<4, false>(c, s.sc, s.ze, w);
-#pragma unroll
-        for (int e = 0; e < 4; ++e)
-            *reinterpret_cast<h16x8*>(&Bs0[buf * B_STAGE + ((bhb * 4 + e) * BN + bn) * 8]) = w[e];
+    auto write_b_fast = [&](const Stage& s, int stage, int q) {
+        *reinterpret_cast<h16x8*>(&Bs[stage * B_STAGE + ((bhb * 2 + q) * BN + bn) * 8]) =
+            dequant_word_int4(s.w[q], stage_negzero(s), stage_scale(s));
     };
+    auto write_b_general = [&](const Stage& s, int stage, int q) {
+        *reinterpret_cast<h16x8*>(&Bs[stage * B_STAGE + ((bhb * 2 + q) * BN + bn) * 8]) =
+            dequant_word_generic4(s.w[q], stage_scale(s).x, -stage_negzero(s).x);
+    };
+
     f32x16 acc[TM][TN];
 #pragma unroll
     for (int i = 0; i < TM; ++i)
@@ -340,95 +345,136 @@ __global__ __launch_bounds__(512) void matmul_kernel_pipe(MatmulArgs a) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-    // fragment addresses (halves, inside a stage) for k slice 0; slice ks adds to kc
+    // fragment addresses (halves, inside a stage); k slice ks selects chunk 2 ks + lane / 32
     int a_frag[TM], b_frag[TN];
 #pragma unroll
-    for (int i = 0; i < TM; ++i) a_frag[i] = (wm0 + i * 32 + (lane & 31)) * BK;
+    for (int i = 0; i < TM; ++i) a_frag[i] = (wm0 + i * 32 + (lane & 31)) * PK;
 #pragma unroll
     for (int j = 0; j < TN; ++j) b_frag[j] = (wn0 + j * 32 + (lane & 31)) * 8;
-    const int a_sw = a_swz(lane & 31);                // rows differ by multiples of 32: same swizzle
-    auto load_frags = [&](int buf, int ks, h16x8 fa[TM], h16x8 fb[TN]) {
+    const int a_sw = (lane >> 2) & 3;                 // row offsets are multiples of 32: same swizzle
+    auto load_frags = [&](int stage, int ks, h16x8 fa[TM], h16x8 fb[TN]) {
         const int kc = 2 * ks + (lane >> 5);
 #pragma unroll
         for (int i = 0; i < TM; ++i)
-            fa[i] = *reinterpret_cast<const h16x8*>(&As0[buf * A_STAGE + a_frag[i] + ((kc ^ a_sw) << 3)]);
+            fa[i] = *reinterpret_cast<const h16x8*>(&As[stage * A_STAGE + a_frag[i] + ((kc ^ a_sw) << 3)]);
 #pragma unroll
         for (int j = 0; j < TN; ++j)
-            fb[j] = *reinterpret_cast<const h16x8*>(&Bs0[buf * B_STAGE + kc * BN * 8 + b_frag[j]]);
+            fb[j] = *reinterpret_cast<const h16x8*>(&Bs[stage * B_STAGE + kc * BN * 8 + b_frag[j]]);
+    };
+    auto mfma_slice = [&](const h16x8 fa[TM], const h16x8 fb[TN]) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[i], fb[j], acc[i][j], 0, 0, 0);
     };
 
-    using True = std::integral_constant<bool, true>;
-    using False = std::integral_constant<bool, false>;
-    const int ktiles = a.K / BK;
+    const int ktiles = a.K / PK;
+    const int last = ktiles - 1;
 
     // Does any (group, column) of this tile use exponent quantisation (scale < 0
     // or NaN)?  One pass over the tile's scales (a few KB); the answer is
     // workgroup-uniform and selects between the pipelined loop, whose decode is
     // the branch-free linear one, and a plain loop with the general decode.
-    __shared__ int any_expo;
+    int& any_expo = *reinterpret_cast<int*>(Bs);          // borrowed before the pipeline starts
+    __syncthreads();
     if (t == 0) any_expo = 0;
     __syncthreads();
     {
         bool bad = false;
-        const int groups = (ktiles + a.group_units - 1) / a.group_units;
+        const int groups = (ktiles + a.group_units * 2 - 1) / (a.group_units * 2);
         for (int g = bhb; g < groups; g += 2) bad |= !(a.scales[(int64_t)g * a.S + bcol] >= (h16)0.0f);
         if (__builtin_amdgcn_ballot_w64(bad) != 0 && lane == 0) any_expo = 1;
     }
     __syncthreads();
+    const bool tile_has_expo = any_expo != 0;
+    __syncthreads();
 
-    if (any_expo == 0) {
-        // One K step: MFMAs on stage `buf`; meanwhile stage buf^1 is filled for the
-        // next step.  A single branch-free body serves every step: near the end
-        // the loads are clamped to the last K step and their results are unused.
-        const int last = ktiles - 1;
-        auto body = [&](int kt, Stage& cur, Stage& nxt, int buf) {
-            load_a(min(kt + 1, last), buf ^ 1);
-            load_b(cur, min(kt + 2, last));
-#pragma unroll
-            for (int ks = 0; ks < 4; ++ks) {
-                h16x8 fa[TM], fb[TN];
-                load_frags(buf, ks, fa, fb);
-                write_b_fast(nxt, buf ^ 1, ks);
-#pragma unroll
-                for (int i = 0; i < TM; ++i)
-#pragma unroll
-                    for (int j = 0; j < TN; ++j)
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+    if (!tile_has_expo) {
+        // Cursor of the weight loads (four K steps ahead of the MFMAs) with the
+        // quantisation group of that step kept by counting instead of dividing.
+        int ld_kt = 0, ld_group = 0, ld_left = a.group_units * 2;
+        auto advance = [&]() {              // one K step forward, clamped at the end
+            if (ld_kt < last) {
+                ++ld_kt;
+                if (--ld_left == 0) { ++ld_group; ld_left = a.group_units * 2; }
             }
-            __syncthreads();      // also waits for this wave's direct-to-LDS loads and LDS writes
         };
-        load_a(0, 0);
-        load_b(st[0], 0);
-        load_b(st[1], min(1, last));
+        Stage r0, r1, r2, r3;
+        AStage ra0, ra1;
+        h16x8 fa[2][TM], fb[2][TN];         // fragments of the current and the next k slice
+        // Step kt with b = kt % 4.  On entry: states and decoded weights of steps
+        // kt, kt+1 are complete in stages b, b+1; ra_wr holds the states and r_dec the
+        // packed weights of step kt+2, which this step moves into stage b+2; the
+        // fragments of slice (kt, 0) are in fa[0] / fb[0].
+        auto body = [&](int kt, int b, AStage& ra_new, const AStage& ra_wr, Stage& r_new, const Stage& r_dec) {
+            load_a(ra_new, min(kt + 3, last));
+            load_b(r_new, ld_kt, ld_group);          // step kt + 4
+            advance();
+            __builtin_amdgcn_sched_barrier(0);       // keep the global loads at the top of the step
 #pragma unroll
-        for (int q = 0; q < 4; ++q) write_b_fast(st[0], 0, q);
+            for (int ks = 0; ks < 2; ++ks) {
+                if (ks == 0) load_frags(b, 1, fa[1], fb[1]);
+                else load_frags((b + 1) & 3, 0, fa[0], fb[0]);
+                write_b_fast(r_dec, (b + 2) & 3, ks);
+                if (ks == 1) write_a(ra_wr, (b + 2) & 3);
+                mfma_slice(fa[ks], fb[ks]);
+                // scheduling template of this k slice: the next slice's fragment reads
+                // first, then every MFMA followed by a few decode instructions, the LDS
+                // stores last
+                __builtin_amdgcn_sched_group_barrier(0x100, TM + TN, 0);
+#pragma unroll
+                for (int e = 0; e < TM * TN; ++e) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x002, TM == 4 ? 3 : 6, 0);
+                }
+                if (ks == 0) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+                else __builtin_amdgcn_sched_group_barrier(0x200, 1 + A_LOADS, 0);
+            }
+            // this step's LDS stores are complete; then all waves meet
+            __builtin_amdgcn_s_waitcnt(0xC07F);      // lgkmcnt(0) only
+            __builtin_amdgcn_s_barrier();
+        };
+        load_a(ra0, 0);
+        load_a(ra1, min(1, last));
+        load_b(r0, ld_kt, ld_group); advance();
+        load_b(r1, ld_kt, ld_group); advance();
+        write_a(ra0, 0);
+        write_a(ra1, 1);
+        load_a(ra0, min(2, last));
+        load_b(r2, ld_kt, ld_group); advance();
+        load_b(r3, ld_kt, ld_group); advance();
+#pragma unroll
+        for (int q = 0; q < 2; ++q) { write_b_fast(r0, 0, q); write_b_fast(r1, 1, q); }
         __syncthreads();
-        int kt = 0;
-        for (; kt + 1 < ktiles; kt += 2) {
-            body(kt, st[0], st[1], 0);
-            body(kt + 1, st[1], st[0], 1);
+        load_frags(0, 0, fa[0], fb[0]);
+        // register sets and LDS stages rotate with periods 2 and 4 (unrolled so
+        // that they are compile-time names)
+        for (int kt = 0; kt < ktiles; kt += 4) {
+            body(kt, 0, ra1, ra0, r0, r2);
+            if (kt + 1 < ktiles) body(kt + 1, 1, ra0, ra1, r1, r3);
+            if (kt + 2 < ktiles) body(kt + 2, 2, ra1, ra0, r2, r0);
+            if (kt + 3 < ktiles) body(kt + 3, 3, ra0, ra1, r3, r1);
         }
-        if (kt < ktiles) body(kt, st[0], st[1], 0);
     } else {
+        Stage r;
+        AStage ra;
+        h16x8 fa[TM], fb[TN];
         for (int kt = 0; kt < ktiles; ++kt) {
-            load_a(kt, 0);
-            load_b(st[0], kt);
-            write_b_general(st[0], 0);
+            load_a(ra, kt);
+            load_b(r, kt, kt / (a.group_units * 2));
+            write_a(ra, 0);
+            write_b_general(r, 0, 0);
+            write_b_general(r, 0, 1);
             __syncthreads();
-#pragma unroll 1
-            for (int ks = 0; ks < 4; ++ks) {
-                h16x8 fa[TM], fb[TN];
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks) {
                 load_frags(0, ks, fa, fb);
-#pragma unroll
-                for (int i = 0; i < TM; ++i)
-#pragma unroll
-                    for (int j = 0; j < TN; ++j)
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+                mfma_slice(fa, fb);
             }
             __syncthreads();
         }
     }
-
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -437,23 +483,28 @@ __global__ __launch_bounds__(512) void matmul_kernel_pipe(MatmulArgs a) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int row = m0 + wm0 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-                if (row < a.M && col < a.S) outs[(int64_t)row * a.S + col] = (h16)acc[i][j][r];
+                outs[(int64_t)row * a.S + col] = (h16)acc[i][j][r];
             }
         }
+}
+
+__global__ __launch_bounds__(512) void matmul_kernel_pipe(MatmulArgs a) {
+    __shared__ __attribute__((aligned(16))) h16 As[4 * 256 * PK];
+    __shared__ __attribute__((aligned(16))) h16 Bs[4 * PK * 256];
+    int bid = blockIdx.x;
+    const int total = a.tiles_m * a.tiles_n;
+    if (total % 8 == 0) bid = (bid % 8) * (total / 8) + bid / 8;     // XCD-aware renumbering
+    const int tile_m = bid % a.tiles_m, tile_n = bid / a.tiles_m;
+    const int64_t boff = blockIdx.z;
+    pipe_tile<4>(a, tile_m * 256, tile_n * 256, a.x + boff * a.M * (int64_t)a.K,
+                 a.outs + boff * a.M * (int64_t)a.S, As, Bs);
 }
 
 static void launch_pipe(MatmulArgs a, int64_t B, hipStream_t st) {
     a.tiles_m = (a.M + 255) / 256;
     a.tiles_n = (a.S + 255) / 256;
     const dim3 grid(a.tiles_m * a.tiles_n, 1, (unsigned)B), block(512);
-    constexpr size_t lds = 2 * (size_t)(256 + 256) * BK * sizeof(h16);
-    static bool attr_set = false;       // the attribute sticks to the function for the whole process
-    if (!attr_set) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(matmul_kernel_pipe),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        attr_set = true;
-    }
-    hipLaunchKernelGGL(matmul_kernel_pipe, grid, block, lds, st, a);
+    hipLaunchKernelGGL(matmul_kernel_pipe, grid, block, 0, st, a);
 }
 
 template <int BITS, bool SPARSE, int BM, int BN, int WM, int WN>
