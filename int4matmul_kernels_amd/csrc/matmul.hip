@@ -252,8 +252,10 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 2) void matmul_kernel(M
         }
 }
 
-// ---- pipelined variant for dense int4: (TM * 64) x 256 tile, 8 waves (2 x 4) of
-// (TM * 32) x 64, K steps of 32, four LDS stages of each operand (128 KB).
+// ---- pipelined variant for dense int4: (TM * 64) x (NW * 64) tile, 2 x NW waves
+// of (TM * 32) x 64, K steps of 32, three LDS stages of each operand.  With
+// NW = 2 (256 x 128 tile, 72 KB of LDS, four waves) two workgroups share a CU
+// and fill each other's barrier and latency bubbles.
 //  * states go global -> registers three steps ahead and are stored to the LDS
 //    stage of step k+2 during step k;
 //  * packed weights go global -> registers four steps ahead and are decoded
@@ -274,55 +276,68 @@ __device__ __forceinline__ h16x8 dequant_word_generic4(uint32_t w, h16 sc, h16 z
     return r;
 }
 
-template <int TM>
+constexpr int P_STAGES = 3;
+
+template <int TM, int NW>
 __device__ __forceinline__ void pipe_tile(const MatmulArgs& a, const int m0, const int s0, const h16* x,
                                           h16* outs, h16* As, h16* Bs) {
-    constexpr int BM = TM * 64, BN = 256, WM = TM * 32, WN = 64, TN = 2;
-    constexpr int A_STAGE = 256 * PK, B_STAGE = PK * BN;           // halves per stage (A sized for TM = 4)
-    constexpr int A_LOADS = TM / 2;                                // direct-to-LDS loads per wave and step
+    constexpr int BM = TM * 64, BN = NW * 64, WM = TM * 32, WN = 64, TN = 2, T = 2 * NW * 64;
+    constexpr int A_STAGE = BM * PK, B_STAGE = PK * BN;            // halves per stage
+    constexpr int A_ROWS = T / 4;                                  // rows covered by one 16-byte load per thread
+    constexpr int A_LOADS = BM / A_ROWS;                           // such loads per thread and step
 
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
-    const int wm0 = (wave >> 2) * WM, wn0 = (wave & 3) * WN;
+    const int wm0 = (wave / NW) * WM, wn0 = (wave % NW) * WN;
 
     // states stage: row m at m * 64 bytes, 16-byte chunk c of the row stored at
     // c ^ ((m >> 2) & 3): sixteen consecutive rows read the same logical chunk
     // from sixteen different bank groups.  Thread t moves chunk t % 4 of rows
-    // t / 4 and t / 4 + 128 through registers.  The tile lies inside the matrix
+    // t / 4 + A_ROWS * i through registers.  The tile lies inside the matrix
     // (launcher's duty).
     struct AStage { u32x4 v[A_LOADS]; };
     const int a_row = t >> 2, a_chunk = t & 3;
-    const h16* a_src = x + (int64_t)(m0 + a_row) * a.K + a_chunk * 8;
-    const int64_t a_row128 = (int64_t)128 * a.K;
-    const int a_dst = a_row * PK + ((a_chunk ^ ((a_row >> 2) & 3)) << 3);       // halves; rows + 128: same swizzle
-    auto load_a = [&](AStage& r, int kt) {
+    // every global address is a workgroup-uniform 64-bit base that moves with the
+    // K step (scalar registers) plus a per-lane 32-bit byte offset that never changes
+    const char* const a_tile = reinterpret_cast<const char*>(x + (int64_t)m0 * a.K);
+    uint32_t a_off[A_LOADS];
 #pragma unroll
-        for (int i = 0; i < A_LOADS; ++i)
-            r.v[i] = *reinterpret_cast<const u32x4*>(a_src + i * a_row128 + kt * PK);
+    for (int i = 0; i < A_LOADS; ++i) a_off[i] = (uint32_t)(((a_row + A_ROWS * i) * a.K + a_chunk * 8) * 2);
+    const int a_dst = a_row * PK + ((a_chunk ^ ((a_row >> 2) & 3)) << 3);       // halves; rows + A_ROWS: same swizzle
+    auto load_a = [&](AStage& r, const char* base) {
+#pragma unroll
+        for (int i = 0; i < A_LOADS; ++i) r.v[i] = *reinterpret_cast<const u32x4*>(base + a_off[i]);
     };
     auto write_a = [&](const AStage& r, int stage) {
 #pragma unroll
         for (int i = 0; i < A_LOADS; ++i)
-            *reinterpret_cast<u32x4*>(&As[stage * A_STAGE + i * 128 * PK + a_dst]) = r.v[i];
+            *reinterpret_cast<u32x4*>(&As[stage * A_STAGE + i * A_ROWS * PK + a_dst]) = r.v[i];
     };
 
     // weights: thread owns column bn and packed rows 2 bhb, 2 bhb + 1 of every K step.
     // scale / zero travel as the aligned 32-bit word that holds the column's half
     // (sub-dword loads make the compiler wait for every outstanding load); `half_sel`
     // replicates the wanted half into both lanes of a packed register.
-    const int bn = t & 255, bhb = t >> 8;
+    const int bn = t % BN, bhb = t / BN;
     const int bcol = s0 + bn;
     struct Stage { uint32_t w[2]; uint32_t sc, ze; };
     const uint32_t half_sel = (bcol & 1) ? 0x03020302u : 0x01000100u;
-    const uint32_t* b_base = a.matrix + (int64_t)bhb * 2 * a.S + bcol;
-    const int64_t b_step = (int64_t)4 * a.S;
-    const h16* sc_base = a.scales + (bcol & ~1);
-    const h16* ze_base = a.zeros + (bcol & ~1);
-    auto load_b = [&](Stage& s, int kt, int group) {
-        const uint32_t* p = b_base + kt * b_step;
-        s.w[0] = p[0];
-        s.w[1] = p[a.S];
-        s.sc = *reinterpret_cast<const uint32_t*>(sc_base + (int64_t)group * a.S);
-        s.ze = *reinterpret_cast<const uint32_t*>(ze_base + (int64_t)group * a.S);
+    const uint32_t b_off0 = (uint32_t)((bhb * 2 * a.S + bcol) * 4), b_off1 = b_off0 + (uint32_t)a.S * 4;
+    const uint32_t sz_off = (uint32_t)((bcol & ~1) * 2);
+    const int64_t b_step = (int64_t)16 * a.S;            // bytes of packed weights per K step (4 rows)
+    const int64_t g_step = (int64_t)2 * a.S;             // bytes of one row of scales / zeros
+    // cursor over K steps: packed-weight rows and the scale / zero row of the step's group
+    struct Cursor { const char* w; const char* sc; const char* ze; int kt, left; };
+    auto cursor_at = [&](int kt) {
+        const int gu = a.group_units * 2, group = kt / gu;
+        return Cursor{reinterpret_cast<const char*>(a.matrix) + kt * b_step,
+                      reinterpret_cast<const char*>(a.scales) + group * g_step,
+                      reinterpret_cast<const char*>(a.zeros) + group * g_step, kt, gu - kt % gu};
+    };
+    auto load_b = [&](Stage& s, const Cursor& c) {
+        s.w[0] = *reinterpret_cast<const uint32_t*>(c.w + b_off0);
+        s.w[1] = *reinterpret_cast<const uint32_t*>(c.w + b_off1);
+        s.sc = *reinterpret_cast<const uint32_t*>(c.sc + sz_off);
+        s.ze = *reinterpret_cast<const uint32_t*>(c.ze + sz_off);
     };
     auto stage_scale = [&](const Stage& s) { return as_h2(__builtin_amdgcn_perm(s.sc, s.sc, half_sel)); };
     auto stage_negzero = [&](const Stage& s) {
@@ -391,42 +406,60 @@ __device__ __forceinline__ void pipe_tile(const MatmulArgs& a, const int m0, con
     __syncthreads();
 
     if (!tile_has_expo) {
-        // Cursor of the weight loads (four K steps ahead of the MFMAs) with the
-        // quantisation group of that step kept by counting instead of dividing.
-        int ld_kt = 0, ld_group = 0, ld_left = a.group_units * 2;
-        auto advance = [&]() {              // one K step forward, clamped at the end
-            if (ld_kt < last) {
-                ++ld_kt;
-                if (--ld_left == 0) { ++ld_group; ld_left = a.group_units * 2; }
-            }
+        // Cursors of the loads: weights run four K steps ahead of the MFMAs, states
+        // three; both stop at the last step (the surplus loads re-read it, unused).
+        Cursor cur = cursor_at(0);
+        // (selects instead of branches: a branch here would split the scheduling
+        // region of the step and invite the compiler to reuse the previous step's
+        // scale / zero registers, which makes the step wait for its newest loads)
+        auto advance = [&]() {
+            const bool more = cur.kt < last;
+            const bool wrap = more && cur.left == 1;
+            cur.kt += more ? 1 : 0;
+            cur.w += more ? b_step : 0;
+            cur.sc += wrap ? g_step : 0;
+            cur.ze += wrap ? g_step : 0;
+            cur.left = wrap ? a.group_units * 2 : cur.left - (more ? 1 : 0);
         };
-        Stage r0, r1, r2, r3;
-        AStage ra0, ra1;
+        const char* a_cur = a_tile;
+        int a_kt = 0;
+        auto advance_a = [&]() {
+            const bool more = a_kt < last;
+            a_kt += more ? 1 : 0;
+            a_cur += more ? PK * 2 : 0;
+        };
+        Stage r[3];
+        AStage ra[2];
         h16x8 fa[2][TM], fb[2][TN];         // fragments of the current and the next k slice
-        // Step kt with b = kt % 4.  On entry: states and decoded weights of steps
-        // kt, kt+1 are complete in stages b, b+1; ra_wr holds the states and r_dec the
-        // packed weights of step kt+2, which this step moves into stage b+2; the
-        // fragments of slice (kt, 0) are in fa[0] / fb[0].
-        auto body = [&](int kt, int b, AStage& ra_new, const AStage& ra_wr, Stage& r_new, const Stage& r_dec) {
-            load_a(ra_new, min(kt + 3, last));
-            load_b(r_new, ld_kt, ld_group);          // step kt + 4
-            advance();
-            __builtin_amdgcn_sched_barrier(0);       // keep the global loads at the top of the step
+        // Step kt, u = kt % 6, stage b = kt % 3.  On entry: states and decoded weights
+        // of steps kt, kt+1 are complete in stages b, b+1; ra[kt % 2] holds the states
+        // and r[(kt+2) % 3] the packed weights of step kt+2, which this step moves
+        // into stage b+2; the fragments of slice (kt, 0) are in fa[0] / fb[0].  The
+        // step loads states kt+3 and weights kt+4 into the register sets it does not use.
+        auto body = [&](int b, AStage& ra_new, const AStage& ra_wr, Stage& r_new, const Stage& r_dec) {
+            const int b1 = (b + 1) % P_STAGES, b2 = (b + 2) % P_STAGES;
 #pragma unroll
             for (int ks = 0; ks < 2; ++ks) {
                 if (ks == 0) load_frags(b, 1, fa[1], fb[1]);
-                else load_frags((b + 1) & 3, 0, fa[0], fb[0]);
-                write_b_fast(r_dec, (b + 2) & 3, ks);
-                if (ks == 1) write_a(ra_wr, (b + 2) & 3);
+                else load_frags(b1, 0, fa[0], fb[0]);
+                if (ks == 0) {
+                    load_a(ra_new, a_cur);             // step kt + 3
+                    load_b(r_new, cur);                // step kt + 4
+                    advance_a();
+                    advance();
+                }
+                write_b_fast(r_dec, b2, ks);
+                if (ks == 1) write_a(ra_wr, b2);
                 mfma_slice(fa[ks], fb[ks]);
                 // scheduling template of this k slice: the next slice's fragment reads
-                // first, then every MFMA followed by a few decode instructions, the LDS
-                // stores last
+                // first, then every MFMA followed by a few decode instructions (and, in
+                // the first slice, one of this step's global loads), the LDS stores last
                 __builtin_amdgcn_sched_group_barrier(0x100, TM + TN, 0);
 #pragma unroll
                 for (int e = 0; e < TM * TN; ++e) {
                     __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
                     __builtin_amdgcn_sched_group_barrier(0x002, TM == 4 ? 3 : 6, 0);
+                    if (ks == 0 && e < A_LOADS + 4) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
                 }
                 if (ks == 0) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
                 else __builtin_amdgcn_sched_group_barrier(0x200, 1 + A_LOADS, 0);
@@ -435,34 +468,35 @@ __device__ __forceinline__ void pipe_tile(const MatmulArgs& a, const int m0, con
             __builtin_amdgcn_s_waitcnt(0xC07F);      // lgkmcnt(0) only
             __builtin_amdgcn_s_barrier();
         };
-        load_a(ra0, 0);
-        load_a(ra1, min(1, last));
-        load_b(r0, ld_kt, ld_group); advance();
-        load_b(r1, ld_kt, ld_group); advance();
-        write_a(ra0, 0);
-        write_a(ra1, 1);
-        load_a(ra0, min(2, last));
-        load_b(r2, ld_kt, ld_group); advance();
-        load_b(r3, ld_kt, ld_group); advance();
+        load_a(ra[0], a_cur); advance_a();
+        load_a(ra[1], a_cur); advance_a();
+        load_b(r[0], cur); advance();
+        load_b(r[1], cur); advance();
+        write_a(ra[0], 0);
+        write_a(ra[1], 1);
+        load_a(ra[0], a_cur); advance_a();              // step 2
 #pragma unroll
-        for (int q = 0; q < 2; ++q) { write_b_fast(r0, 0, q); write_b_fast(r1, 1, q); }
+        for (int q = 0; q < 2; ++q) { write_b_fast(r[0], 0, q); write_b_fast(r[1], 1, q); }
+        load_b(r[2], cur); advance();                   // step 2
+        load_b(r[0], cur); advance();                   // step 3
         __syncthreads();
         load_frags(0, 0, fa[0], fb[0]);
-        // register sets and LDS stages rotate with periods 2 and 4 (unrolled so
-        // that they are compile-time names)
-        for (int kt = 0; kt < ktiles; kt += 4) {
-            body(kt, 0, ra1, ra0, r0, r2);
-            if (kt + 1 < ktiles) body(kt + 1, 1, ra0, ra1, r1, r3);
-            if (kt + 2 < ktiles) body(kt + 2, 2, ra1, ra0, r2, r0);
-            if (kt + 3 < ktiles) body(kt + 3, 3, ra0, ra1, r3, r1);
+        // LDS stages and weight registers rotate with period 3, state registers with
+        // period 2: six steps per trip, unrolled so that all of them are compile-time names
+        for (int kt = 0; kt < ktiles; kt += 6) {
+#pragma unroll
+            for (int u = 0; u < 6; ++u) {
+                if (u > 0 && kt + u >= ktiles) break;
+                body(u % 3, ra[(u + 1) % 2], ra[u % 2], r[(u + 1) % 3], r[(u + 2) % 3]);
+            }
         }
     } else {
         Stage r;
         AStage ra;
         h16x8 fa[TM], fb[TN];
         for (int kt = 0; kt < ktiles; ++kt) {
-            load_a(ra, kt);
-            load_b(r, kt, kt / (a.group_units * 2));
+            load_a(ra, a_tile + kt * (PK * 2));
+            load_b(r, cursor_at(kt));
             write_a(ra, 0);
             write_b_general(r, 0, 0);
             write_b_general(r, 0, 1);
@@ -488,23 +522,26 @@ __device__ __forceinline__ void pipe_tile(const MatmulArgs& a, const int m0, con
         }
 }
 
-__global__ __launch_bounds__(512) void matmul_kernel_pipe(MatmulArgs a) {
-    __shared__ __attribute__((aligned(16))) h16 As[4 * 256 * PK];
-    __shared__ __attribute__((aligned(16))) h16 Bs[4 * PK * 256];
+template <int NW>
+__global__ __launch_bounds__(NW * 128, NW == 2 ? 2 : 1) void matmul_kernel_pipe(MatmulArgs a) {
+    constexpr int BM = 256, BN = NW * 64;
+    __shared__ __attribute__((aligned(16))) h16 As[P_STAGES * BM * PK];
+    __shared__ __attribute__((aligned(16))) h16 Bs[P_STAGES * PK * BN];
     int bid = blockIdx.x;
     const int total = a.tiles_m * a.tiles_n;
     if (total % 8 == 0) bid = (bid % 8) * (total / 8) + bid / 8;     // XCD-aware renumbering
     const int tile_m = bid % a.tiles_m, tile_n = bid / a.tiles_m;
     const int64_t boff = blockIdx.z;
-    pipe_tile<4>(a, tile_m * 256, tile_n * 256, a.x + boff * a.M * (int64_t)a.K,
-                 a.outs + boff * a.M * (int64_t)a.S, As, Bs);
+    pipe_tile<4, NW>(a, tile_m * BM, tile_n * BN, a.x + boff * a.M * (int64_t)a.K,
+                     a.outs + boff * a.M * (int64_t)a.S, As, Bs);
 }
 
+template <int NW>
 static void launch_pipe(MatmulArgs a, int64_t B, hipStream_t st) {
-    a.tiles_m = (a.M + 255) / 256;
-    a.tiles_n = (a.S + 255) / 256;
-    const dim3 grid(a.tiles_m * a.tiles_n, 1, (unsigned)B), block(512);
-    hipLaunchKernelGGL(matmul_kernel_pipe, grid, block, 0, st, a);
+    a.tiles_m = a.M / 256;
+    a.tiles_n = a.S / (NW * 64);
+    const dim3 grid(a.tiles_m * a.tiles_n, 1, (unsigned)B), block(NW * 128);
+    hipLaunchKernelGGL(matmul_kernel_pipe<NW>, grid, block, 0, st, a);
 }
 
 template <int BITS, bool SPARSE, int BM, int BN, int WM, int WN>
@@ -522,7 +559,7 @@ static void launch(const MatmulArgs& a, int64_t B, hipStream_t st) {
     // 128 x 128 tiles for narrow outputs or few rows
     int variant = (int)tuning(TUNE_MM_VARIANT);
     const bool pipe_ok = BITS == 4 && !SPARSE && a.M % 256 == 0 && a.S % 256 == 0;
-    if (variant == 5 && !pipe_ok) variant = 0;
+    if ((variant == 5 || variant == 6) && !pipe_ok) variant = 0;
     if (variant == 0) {
         if (pipe_ok) variant = 5;
         else if (a.M > 128 && a.S >= 256) variant = 3;
@@ -532,7 +569,10 @@ static void launch(const MatmulArgs& a, int64_t B, hipStream_t st) {
     else if (variant == 2) launch_tile<BITS, SPARSE, 128, 256, 64, 128>(a, B, st);
     else if (variant == 3) launch_tile<BITS, SPARSE, 128, 256, 128, 64>(a, B, st);
     else if (variant == 4) launch_tile<BITS, SPARSE, 256, 256, 128, 64>(a, B, st);
-    else if constexpr (BITS == 4 && !SPARSE) launch_pipe(a, B, st);
+    else if constexpr (BITS == 4 && !SPARSE) {
+        if (variant == 6) launch_pipe<4>(a, B, st);
+        else launch_pipe<2>(a, B, st);
+    }
 }
 
 }  // namespace i4
