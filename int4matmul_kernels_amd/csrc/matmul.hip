@@ -269,16 +269,54 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 2) void matmul_kernel(M
 // groups takes a plain loop with the general decode instead.
 constexpr int PK = 32;            // K per step of the pipelined kernel
 
-__device__ __forceinline__ h16x8 dequant_word_generic4(uint32_t w, h16 sc, h16 ze) {
+// One 16-byte chunk = 8 consecutive k of one column.  `bits` holds its 8 codes,
+// LSB first, BITS bits apart (bits above 8 * BITS are ignored).
+template <int BITS>
+__device__ __forceinline__ h16x8 dequant_chunk_generic(uint32_t bits, h16 sc, h16 ze) {
     h16x8 r;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) r[e] = dequant_code<4>((w >> (4 * e)) & 15u, sc, ze);
+    for (int e = 0; e < 8; ++e) r[e] = dequant_code<BITS>((bits >> (BITS * e)) & ((1u << BITS) - 1u), sc, ze);
     return r;
 }
 
+// Linear-mode fast decode of such a chunk, bit-exact.  The two codes of a pair
+// are brought to the low bits of the two halves of a register; mask-and-OR with
+// a magic exponent turns them into {2^a + q_even, 2^b + q_odd}, whose offsets
+// are then subtracted exactly before the reference's two roundings.
+template <int BITS>
+__device__ __forceinline__ h16x8 dequant_chunk_fast(uint32_t bits, h16x2 negz, h16x2 s2) {
+    if constexpr (BITS == 4) {
+        return dequant_word_int4(bits, negz, s2);
+    } else {
+        // int2: pair j = bits 4j .. 4j+3 of the 16 code bits, replicated into both halves:
+        //       low half keeps bits 0-1 (ulp 1 at 2^10), high half bits 2-3 (ulp 1/4 at 2^8).
+        // int3: pair j = bits 6j .. 6j+5: low half bits 0-2 (2^10), high half bits 3-5 (ulp 1/8 at 2^7).
+        constexpr uint32_t MSK = BITS == 2 ? 0x000C0003u : 0x00380007u;
+        constexpr uint32_t MAGIC = BITS == 2 ? 0x5C006400u : 0x58006400u;
+        const h16x2 unmagic = {(h16)-1024.0f, BITS == 2 ? (h16)-256.0f : (h16)-128.0f};
+        u32x4 r;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t u = bits >> (2 * BITS * j);
+            const uint32_t v = (u << 16) | u;
+            h16x2 q = as_h2((v & MSK) | MAGIC) + unmagic;      // exact: {q_even, q_odd}
+            h16x2 d = q + negz;                                // fp16 subtract, one rounding
+            r[j] = as_u32(d * s2);                             // fp16 multiply, one rounding
+        }
+        return bitcast<h16x8>(r);
+    }
+}
+
+// Per-format constants of the pipelined kernel: packed rows per 32-row block and
+// the number of packed words a thread loads per K step for its two chunks.
+template <int BITS> struct PipeFmt;
+template <> struct PipeFmt<4> { static constexpr int ROWS = 4, NWORDS = 2; };
+template <> struct PipeFmt<3> { static constexpr int ROWS = 3, NWORDS = 2; };
+template <> struct PipeFmt<2> { static constexpr int ROWS = 2, NWORDS = 1; };
+
 constexpr int P_STAGES = 3;
 
-template <int TM, int NW>
+template <int BITS, int TM, int NW>
 __device__ __forceinline__ void pipe_tile(const MatmulArgs& a, const int m0, const int s0, const h16* x,
                                           h16* outs, h16* As, h16* Bs) {
     constexpr int BM = TM * 64, BN = NW * 64, WM = TM * 32, WN = 64, TN = 2, T = 2 * NW * 64;
@@ -317,13 +355,21 @@ __device__ __forceinline__ void pipe_tile(const MatmulArgs& a, const int m0, con
     // scale / zero travel as the aligned 32-bit word that holds the column's half
     // (sub-dword loads make the compiler wait for every outstanding load); `half_sel`
     // replicates the wanted half into both lanes of a packed register.
+    // Thread (bn, bhb) decodes rows 16 bhb .. 16 bhb + 15 of the step's 32-row block:
+    // int4 words 2 bhb, 2 bhb + 1; int2 word bhb; int3 words bhb, bhb + 1 (bits
+    // 48 bhb .. 48 bhb + 47 of the block's 96-bit stream).
+    using F = PipeFmt<BITS>;
+    constexpr int NWORDS = F::NWORDS;
     const int bn = t % BN, bhb = t / BN;
     const int bcol = s0 + bn;
-    struct Stage { uint32_t w[2]; uint32_t sc, ze; };
+    struct Stage { uint32_t w[NWORDS]; uint32_t sc, ze; };
     const uint32_t half_sel = (bcol & 1) ? 0x03020302u : 0x01000100u;
-    const uint32_t b_off0 = (uint32_t)((bhb * 2 * a.S + bcol) * 4), b_off1 = b_off0 + (uint32_t)a.S * 4;
+    uint32_t b_off[NWORDS];
+#pragma unroll
+    for (int i = 0; i < NWORDS; ++i)
+        b_off[i] = (uint32_t)((((BITS == 4 ? 2 * bhb : bhb) + i) * a.S + bcol) * 4);
     const uint32_t sz_off = (uint32_t)((bcol & ~1) * 2);
-    const int64_t b_step = (int64_t)16 * a.S;            // bytes of packed weights per K step (4 rows)
+    const int64_t b_step = (int64_t)(F::ROWS * 4) * a.S;  // bytes of packed weights per K step
     const int64_t g_step = (int64_t)2 * a.S;             // bytes of one row of scales / zeros
     // cursor over K steps: packed-weight rows and the scale / zero row of the step's group
     struct Cursor { const char* w; const char* sc; const char* ze; int kt, left; };
@@ -334,8 +380,8 @@ __device__ __forceinline__ void pipe_tile(const MatmulArgs& a, const int m0, con
                       reinterpret_cast<const char*>(a.zeros) + group * g_step, kt, gu - kt % gu};
     };
     auto load_b = [&](Stage& s, const Cursor& c) {
-        s.w[0] = *reinterpret_cast<const uint32_t*>(c.w + b_off0);
-        s.w[1] = *reinterpret_cast<const uint32_t*>(c.w + b_off1);
+#pragma unroll
+        for (int i = 0; i < NWORDS; ++i) s.w[i] = *reinterpret_cast<const uint32_t*>(c.w + b_off[i]);
         s.sc = *reinterpret_cast<const uint32_t*>(c.sc + sz_off);
         s.ze = *reinterpret_cast<const uint32_t*>(c.ze + sz_off);
     };
@@ -343,13 +389,20 @@ __device__ __forceinline__ void pipe_tile(const MatmulArgs& a, const int m0, con
     auto stage_negzero = [&](const Stage& s) {
         return as_h2(__builtin_amdgcn_perm(s.ze, s.ze, half_sel) ^ 0x80008000u);
     };
+    // the 8 codes of the thread's chunk q (rows 16 bhb + 8 q .. + 7), LSB first
+    const int i3_shift = 16 * bhb;
+    auto chunk_bits = [&](const Stage& s, int q) -> uint32_t {
+        if constexpr (BITS == 4) return s.w[q];
+        else if constexpr (BITS == 2) return q ? s.w[0] >> 16 : s.w[0];
+        else return (uint32_t)((((uint64_t)s.w[1] << 32) | s.w[0]) >> (i3_shift + 24 * q));
+    };
     auto write_b_fast = [&](const Stage& s, int stage, int q) {
         *reinterpret_cast<h16x8*>(&Bs[stage * B_STAGE + ((bhb * 2 + q) * BN + bn) * 8]) =
-            dequant_word_int4(s.w[q], stage_negzero(s), stage_scale(s));
+            dequant_chunk_fast<BITS>(chunk_bits(s, q), stage_negzero(s), stage_scale(s));
     };
     auto write_b_general = [&](const Stage& s, int stage, int q) {
         *reinterpret_cast<h16x8*>(&Bs[stage * B_STAGE + ((bhb * 2 + q) * BN + bn) * 8]) =
-            dequant_word_generic4(s.w[q], stage_scale(s).x, -stage_negzero(s).x);
+            dequant_chunk_generic<BITS>(chunk_bits(s, q), stage_scale(s).x, -stage_negzero(s).x);
     };
 
     f32x16 acc[TM][TN];
@@ -459,7 +512,7 @@ __device__ __forceinline__ void pipe_tile(const MatmulArgs& a, const int m0, con
                 for (int e = 0; e < TM * TN; ++e) {
                     __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
                     __builtin_amdgcn_sched_group_barrier(0x002, TM == 4 ? 3 : 6, 0);
-                    if (ks == 0 && e < A_LOADS + 4) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+                    if (ks == 0 && e < A_LOADS + NWORDS + 2) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
                 }
                 if (ks == 0) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
                 else __builtin_amdgcn_sched_group_barrier(0x200, 1 + A_LOADS, 0);
@@ -522,7 +575,7 @@ __device__ __forceinline__ void pipe_tile(const MatmulArgs& a, const int m0, con
         }
 }
 
-template <int NW>
+template <int BITS, int NW>
 __global__ __launch_bounds__(NW * 128, NW == 2 ? 2 : 1) void matmul_kernel_pipe(MatmulArgs a) {
     constexpr int BM = 256, BN = NW * 64;
     __shared__ __attribute__((aligned(16))) h16 As[P_STAGES * BM * PK];
@@ -532,16 +585,16 @@ __global__ __launch_bounds__(NW * 128, NW == 2 ? 2 : 1) void matmul_kernel_pipe(
     if (total % 8 == 0) bid = (bid % 8) * (total / 8) + bid / 8;     // XCD-aware renumbering
     const int tile_m = bid % a.tiles_m, tile_n = bid / a.tiles_m;
     const int64_t boff = blockIdx.z;
-    pipe_tile<4, NW>(a, tile_m * BM, tile_n * BN, a.x + boff * a.M * (int64_t)a.K,
+    pipe_tile<BITS, 4, NW>(a, tile_m * BM, tile_n * BN, a.x + boff * a.M * (int64_t)a.K,
                      a.outs + boff * a.M * (int64_t)a.S, As, Bs);
 }
 
-template <int NW>
+template <int BITS, int NW>
 static void launch_pipe(MatmulArgs a, int64_t B, hipStream_t st) {
     a.tiles_m = a.M / 256;
     a.tiles_n = a.S / (NW * 64);
     const dim3 grid(a.tiles_m * a.tiles_n, 1, (unsigned)B), block(NW * 128);
-    hipLaunchKernelGGL(matmul_kernel_pipe<NW>, grid, block, 0, st, a);
+    hipLaunchKernelGGL((matmul_kernel_pipe<BITS, NW>), grid, block, 0, st, a);
 }
 
 template <int BITS, bool SPARSE, int BM, int BN, int WM, int WN>
@@ -554,14 +607,19 @@ static void launch_tile(MatmulArgs a, int64_t B, hipStream_t st) {
 
 template <int BITS, bool SPARSE>
 static void launch(const MatmulArgs& a, int64_t B, hipStream_t st) {
-    // variant 0 = automatic: the pipelined 256 x 256 kernel where it applies
-    // (dense int4, tile-aligned M and S), otherwise 128 x 256 tiles, and
-    // 128 x 128 tiles for narrow outputs or few rows
+    // variant 0 = automatic.  Dense formats with tile-aligned shapes take the
+    // pipelined kernel: 256 x 128 tiles (two workgroups per CU) when there are
+    // enough of them to keep every CU at two, 256 x 256 tiles (one eight-wave
+    // workgroup per CU) for smaller grids.  Everything else: 128 x 256 tiles, and
+    // 128 x 128 for narrow outputs or few rows.
     int variant = (int)tuning(TUNE_MM_VARIANT);
-    const bool pipe_ok = BITS == 4 && !SPARSE && a.M % 256 == 0 && a.S % 256 == 0;
-    if ((variant == 5 || variant == 6) && !pipe_ok) variant = 0;
+    const bool pipe2_ok = !SPARSE && a.M % 256 == 0 && a.S % 128 == 0;
+    const bool pipe4_ok = !SPARSE && a.M % 256 == 0 && a.S % 256 == 0;
+    if ((variant == 5 && !pipe2_ok) || (variant == 6 && !pipe4_ok)) variant = 0;
     if (variant == 0) {
-        if (pipe_ok) variant = 5;
+        const int64_t tiles4 = (int64_t)(a.M / 256) * (a.S / 256) * B;
+        if (pipe4_ok && tiles4 <= 384) variant = 6;
+        else if (pipe2_ok) variant = 5;
         else if (a.M > 128 && a.S >= 256) variant = 3;
         else variant = 1;
     }
@@ -569,9 +627,9 @@ static void launch(const MatmulArgs& a, int64_t B, hipStream_t st) {
     else if (variant == 2) launch_tile<BITS, SPARSE, 128, 256, 64, 128>(a, B, st);
     else if (variant == 3) launch_tile<BITS, SPARSE, 128, 256, 128, 64>(a, B, st);
     else if (variant == 4) launch_tile<BITS, SPARSE, 256, 256, 128, 64>(a, B, st);
-    else if constexpr (BITS == 4 && !SPARSE) {
-        if (variant == 6) launch_pipe<4>(a, B, st);
-        else launch_pipe<2>(a, B, st);
+    else if constexpr (!SPARSE) {
+        if (variant == 6) launch_pipe<BITS, 4>(a, B, st);
+        else launch_pipe<BITS, 2>(a, B, st);
     }
 }
 
