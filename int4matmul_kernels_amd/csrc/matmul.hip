@@ -298,7 +298,7 @@ __device__ __forceinline__ h16x8 dequant_chunk_fast(uint32_t bits, h16x2 negz, h
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const uint32_t u = bits >> (2 * BITS * j);
-            const uint32_t v = (u << 16) | u;
+            const uint32_t v = __builtin_amdgcn_perm(u, u, 0x01000100u);     // low 16 bits in both halves
             h16x2 q = as_h2((v & MSK) | MAGIC) + unmagic;      // exact: {q_even, q_odd}
             h16x2 d = q + negz;                                // fp16 subtract, one rounding
             r[j] = as_u32(d * s2);                             // fp16 multiply, one rounding
