@@ -307,18 +307,74 @@ __device__ __forceinline__ h16x8 dequant_chunk_fast(uint32_t bits, h16x2 negz, h
     }
 }
 
+// 16:32 sparse int4.  `v` holds the (up to 8) kept codes of one 8-row chunk as
+// consecutive nibbles, `m8` the chunk's mask bits.  A 256-entry table in LDS
+// (8 words per mask byte: four words of per-half keep masks, two v_perm
+// selectors) spreads the kept codes to their rows: the even / odd nibbles are
+// separated into bytes, v_perm picks for every row the byte of its rank, a
+// second v_perm widens byte pairs to {0x6400 | q, 0x6400 | q'}.  Dropped rows
+// are cleared at the end, so they are exactly zero.
+constexpr int SPARSE_LUT_WORDS = 256 * 8;
+
+__device__ __forceinline__ void sparse_lut_entry(uint32_t e, uint32_t out[8]) {
+    uint32_t sel[2] = {0, 0}, hm[4] = {0, 0, 0, 0};
+    uint32_t rank = 0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const bool kept = (e >> i) & 1u;
+        const uint32_t byte = kept ? ((rank & 1u) ? 4u + (rank >> 1) : (rank >> 1)) : 0x0Cu;
+        sel[i >> 2] |= byte << (8 * (i & 3));
+        if (kept) { hm[i >> 1] |= 0xFFFFu << (16 * (i & 1)); ++rank; }
+    }
+    out[0] = hm[0]; out[1] = hm[1]; out[2] = hm[2]; out[3] = hm[3];
+    out[4] = sel[0]; out[5] = sel[1]; out[6] = 0; out[7] = 0;
+}
+
+__device__ __forceinline__ h16x8 dequant_chunk_sparse_fast(uint32_t v, uint32_t m8, const uint32_t* lut,
+                                                           h16x2 negz, h16x2 s2) {
+    const u32x4 keep = *reinterpret_cast<const u32x4*>(lut + m8 * 8);
+    const u32x2 sel = *reinterpret_cast<const u32x2*>(lut + m8 * 8 + 4);
+    const uint32_t even = v & 0x0F0F0F0Fu, odd = (v >> 4) & 0x0F0F0F0Fu;
+    const uint32_t c03 = __builtin_amdgcn_perm(odd, even, sel.x);       // codes of rows 0..3, one per byte
+    const uint32_t c47 = __builtin_amdgcn_perm(odd, even, sel.y);
+    const uint32_t MAGIC = 0x64006400u;
+    const uint32_t h[4] = {__builtin_amdgcn_perm(c03, MAGIC, 0x01050104u), __builtin_amdgcn_perm(c03, MAGIC, 0x01070106u),
+                           __builtin_amdgcn_perm(c47, MAGIC, 0x01050104u), __builtin_amdgcn_perm(c47, MAGIC, 0x01070106u)};
+    const h16x2 unmagic = {(h16)-1024.0f, (h16)-1024.0f};
+    u32x4 r;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        h16x2 q = as_h2(h[i]) + unmagic;       // exact
+        h16x2 d = q + negz;                    // fp16 subtract, one rounding
+        r[i] = as_u32(d * s2) & keep[i];       // fp16 multiply, one rounding; dropped rows -> +0
+    }
+    return bitcast<h16x8>(r);
+}
+
+__device__ __forceinline__ h16x8 dequant_chunk_sparse_generic(uint32_t v, uint32_t m8, h16 sc, h16 ze) {
+    h16x8 r;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        const bool kept = (m8 >> e) & 1u;
+        r[e] = kept ? dequant_code<4>(v & 15u, sc, ze) : (h16)0.0f;
+        v >>= kept ? 4 : 0;
+    }
+    return r;
+}
+
 // Per-format constants of the pipelined kernel: packed rows per 32-row block and
 // the number of packed words a thread loads per K step for its two chunks.
-template <int BITS> struct PipeFmt;
-template <> struct PipeFmt<4> { static constexpr int ROWS = 4, NWORDS = 2; };
-template <> struct PipeFmt<3> { static constexpr int ROWS = 3, NWORDS = 2; };
-template <> struct PipeFmt<2> { static constexpr int ROWS = 2, NWORDS = 1; };
+template <int BITS, bool SPARSE> struct PipeFmt;
+template <> struct PipeFmt<4, false> { static constexpr int ROWS = 4, NWORDS = 2; };
+template <> struct PipeFmt<3, false> { static constexpr int ROWS = 3, NWORDS = 2; };
+template <> struct PipeFmt<2, false> { static constexpr int ROWS = 2, NWORDS = 1; };
+template <> struct PipeFmt<4, true> { static constexpr int ROWS = 2, NWORDS = 2; };
 
 constexpr int P_STAGES = 3;
 
-template <int BITS, int TM, int NW>
+template <int BITS, bool SPARSE, int TM, int NW>
 __device__ __forceinline__ void pipe_tile(const MatmulArgs& a, const int m0, const int s0, const h16* x,
-                                          h16* outs, h16* As, h16* Bs) {
+                                          h16* outs, h16* As, h16* Bs, uint32_t* lut) {
     constexpr int BM = TM * 64, BN = NW * 64, WM = TM * 32, WN = 64, TN = 2, T = 2 * NW * 64;
     constexpr int A_STAGE = BM * PK, B_STAGE = PK * BN;            // halves per stage
     constexpr int A_ROWS = T / 4;                                  // rows covered by one 16-byte load per thread
@@ -357,31 +413,36 @@ __device__ __forceinline__ void pipe_tile(const MatmulArgs& a, const int m0, con
     // replicates the wanted half into both lanes of a packed register.
     // Thread (bn, bhb) decodes rows 16 bhb .. 16 bhb + 15 of the step's 32-row block:
     // int4 words 2 bhb, 2 bhb + 1; int2 word bhb; int3 words bhb, bhb + 1 (bits
-    // 48 bhb .. 48 bhb + 47 of the block's 96-bit stream).
-    using F = PipeFmt<BITS>;
+    // 48 bhb .. 48 bhb + 47 of the block's 96-bit stream); 16:32 sparse: both words
+    // and the mask word of the block.
+    using F = PipeFmt<BITS, SPARSE>;
     constexpr int NWORDS = F::NWORDS;
     const int bn = t % BN, bhb = t / BN;
     const int bcol = s0 + bn;
-    struct Stage { uint32_t w[NWORDS]; uint32_t sc, ze; };
+    struct Stage { uint32_t w[NWORDS]; uint32_t m; uint32_t sc, ze; };
     const uint32_t half_sel = (bcol & 1) ? 0x03020302u : 0x01000100u;
     uint32_t b_off[NWORDS];
 #pragma unroll
     for (int i = 0; i < NWORDS; ++i)
-        b_off[i] = (uint32_t)((((BITS == 4 ? 2 * bhb : bhb) + i) * a.S + bcol) * 4);
+        b_off[i] = (uint32_t)((((SPARSE ? 0 : BITS == 4 ? 2 * bhb : bhb) + i) * a.S + bcol) * 4);
+    const uint32_t m_off = (uint32_t)(bcol * 4);
+    const int64_t m_step = (int64_t)4 * a.S;             // bytes of one row of mask words
     const uint32_t sz_off = (uint32_t)((bcol & ~1) * 2);
     const int64_t b_step = (int64_t)(F::ROWS * 4) * a.S;  // bytes of packed weights per K step
     const int64_t g_step = (int64_t)2 * a.S;             // bytes of one row of scales / zeros
     // cursor over K steps: packed-weight rows and the scale / zero row of the step's group
-    struct Cursor { const char* w; const char* sc; const char* ze; int kt, left; };
+    struct Cursor { const char* w; const char* m; const char* sc; const char* ze; int kt, left; };
     auto cursor_at = [&](int kt) {
         const int gu = a.group_units * 2, group = kt / gu;
         return Cursor{reinterpret_cast<const char*>(a.matrix) + kt * b_step,
+                      reinterpret_cast<const char*>(a.mask) + (SPARSE ? kt * m_step : 0),
                       reinterpret_cast<const char*>(a.scales) + group * g_step,
                       reinterpret_cast<const char*>(a.zeros) + group * g_step, kt, gu - kt % gu};
     };
     auto load_b = [&](Stage& s, const Cursor& c) {
 #pragma unroll
         for (int i = 0; i < NWORDS; ++i) s.w[i] = *reinterpret_cast<const uint32_t*>(c.w + b_off[i]);
+        if constexpr (SPARSE) s.m = *reinterpret_cast<const uint32_t*>(c.m + m_off);
         s.sc = *reinterpret_cast<const uint32_t*>(c.sc + sz_off);
         s.ze = *reinterpret_cast<const uint32_t*>(c.ze + sz_off);
     };
@@ -396,13 +457,38 @@ __device__ __forceinline__ void pipe_tile(const MatmulArgs& a, const int m0, con
         else if constexpr (BITS == 2) return q ? s.w[0] >> 16 : s.w[0];
         else return (uint32_t)((((uint64_t)s.w[1] << 32) | s.w[0]) >> (i3_shift + 24 * q));
     };
+    // 16:32 sparse: mask bits of chunk q and its kept codes as consecutive nibbles.
+    // The codes of rows before the chunk are skipped by a right shift of 4 bits
+    // each (done in two halves: the total can reach 64).
+    auto sparse_chunk = [&](const Stage& s, int q, uint32_t& v, uint32_t& m8) {
+        const uint32_t m16 = (s.m >> (16 * bhb)) & 0xFFFFu;
+        uint32_t skip = bhb ? __builtin_popcount(s.m & 0xFFFFu) : 0;
+        if (q) skip += __builtin_popcount(m16 & 0xFFu);
+        m8 = (m16 >> (8 * q)) & 0xFFu;
+        const uint64_t st = ((uint64_t)s.w[1] << 32) | s.w[0];
+        v = (uint32_t)((st >> (2 * skip)) >> (2 * skip));
+    };
     auto write_b_fast = [&](const Stage& s, int stage, int q) {
-        *reinterpret_cast<h16x8*>(&Bs[stage * B_STAGE + ((bhb * 2 + q) * BN + bn) * 8]) =
-            dequant_chunk_fast<BITS>(chunk_bits(s, q), stage_negzero(s), stage_scale(s));
+        h16x8 w;
+        if constexpr (SPARSE) {
+            uint32_t v, m8;
+            sparse_chunk(s, q, v, m8);
+            w = dequant_chunk_sparse_fast(v, m8, lut, stage_negzero(s), stage_scale(s));
+        } else {
+            w = dequant_chunk_fast<BITS>(chunk_bits(s, q), stage_negzero(s), stage_scale(s));
+        }
+        *reinterpret_cast<h16x8*>(&Bs[stage * B_STAGE + ((bhb * 2 + q) * BN + bn) * 8]) = w;
     };
     auto write_b_general = [&](const Stage& s, int stage, int q) {
-        *reinterpret_cast<h16x8*>(&Bs[stage * B_STAGE + ((bhb * 2 + q) * BN + bn) * 8]) =
-            dequant_chunk_generic<BITS>(chunk_bits(s, q), stage_scale(s).x, -stage_negzero(s).x);
+        h16x8 w;
+        if constexpr (SPARSE) {
+            uint32_t v, m8;
+            sparse_chunk(s, q, v, m8);
+            w = dequant_chunk_sparse_generic(v, m8, stage_scale(s).x, -stage_negzero(s).x);
+        } else {
+            w = dequant_chunk_generic<BITS>(chunk_bits(s, q), stage_scale(s).x, -stage_negzero(s).x);
+        }
+        *reinterpret_cast<h16x8*>(&Bs[stage * B_STAGE + ((bhb * 2 + q) * BN + bn) * 8]) = w;
     };
 
     f32x16 acc[TM][TN];
@@ -446,6 +532,14 @@ __device__ __forceinline__ void pipe_tile(const MatmulArgs& a, const int m0, con
     // the branch-free linear one, and a plain loop with the general decode.
     int& any_expo = *reinterpret_cast<int*>(Bs);          // borrowed before the pipeline starts
     __syncthreads();
+    if constexpr (SPARSE) {
+        if (t < 256) {
+            uint32_t e[8];
+            sparse_lut_entry(t, e);
+            *reinterpret_cast<u32x4*>(lut + t * 8) = u32x4{e[0], e[1], e[2], e[3]};
+            *reinterpret_cast<u32x4*>(lut + t * 8 + 4) = u32x4{e[4], e[5], e[6], e[7]};
+        }
+    }
     if (t == 0) any_expo = 0;
     __syncthreads();
     {
@@ -470,6 +564,7 @@ __device__ __forceinline__ void pipe_tile(const MatmulArgs& a, const int m0, con
             const bool wrap = more && cur.left == 1;
             cur.kt += more ? 1 : 0;
             cur.w += more ? b_step : 0;
+            if constexpr (SPARSE) cur.m += more ? m_step : 0;
             cur.sc += wrap ? g_step : 0;
             cur.ze += wrap ? g_step : 0;
             cur.left = wrap ? a.group_units * 2 : cur.left - (more ? 1 : 0);
@@ -507,12 +602,12 @@ __device__ __forceinline__ void pipe_tile(const MatmulArgs& a, const int m0, con
                 // scheduling template of this k slice: the next slice's fragment reads
                 // first, then every MFMA followed by a few decode instructions (and, in
                 // the first slice, one of this step's global loads), the LDS stores last
-                __builtin_amdgcn_sched_group_barrier(0x100, TM + TN, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, TM + TN + (SPARSE ? 2 : 0), 0);
 #pragma unroll
                 for (int e = 0; e < TM * TN; ++e) {
                     __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
                     __builtin_amdgcn_sched_group_barrier(0x002, TM == 4 ? 3 : 6, 0);
-                    if (ks == 0 && e < A_LOADS + NWORDS + 2) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+                    if (ks == 0 && e < A_LOADS + NWORDS + (SPARSE ? 3 : 2)) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
                 }
                 if (ks == 0) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
                 else __builtin_amdgcn_sched_group_barrier(0x200, 1 + A_LOADS, 0);
@@ -575,26 +670,27 @@ __device__ __forceinline__ void pipe_tile(const MatmulArgs& a, const int m0, con
         }
 }
 
-template <int BITS, int NW>
+template <int BITS, bool SPARSE, int NW>
 __global__ __launch_bounds__(NW * 128, NW == 2 ? 2 : 1) void matmul_kernel_pipe(MatmulArgs a) {
     constexpr int BM = 256, BN = NW * 64;
     __shared__ __attribute__((aligned(16))) h16 As[P_STAGES * BM * PK];
     __shared__ __attribute__((aligned(16))) h16 Bs[P_STAGES * PK * BN];
+    __shared__ __attribute__((aligned(16))) uint32_t Lut[SPARSE ? SPARSE_LUT_WORDS : 4];
     int bid = blockIdx.x;
     const int total = a.tiles_m * a.tiles_n;
     if (total % 8 == 0) bid = (bid % 8) * (total / 8) + bid / 8;     // XCD-aware renumbering
     const int tile_m = bid % a.tiles_m, tile_n = bid / a.tiles_m;
     const int64_t boff = blockIdx.z;
-    pipe_tile<BITS, 4, NW>(a, tile_m * BM, tile_n * BN, a.x + boff * a.M * (int64_t)a.K,
-                     a.outs + boff * a.M * (int64_t)a.S, As, Bs);
+    pipe_tile<BITS, SPARSE, 4, NW>(a, tile_m * BM, tile_n * BN, a.x + boff * a.M * (int64_t)a.K,
+                                   a.outs + boff * a.M * (int64_t)a.S, As, Bs, Lut);
 }
 
-template <int BITS, int NW>
+template <int BITS, bool SPARSE, int NW>
 static void launch_pipe(MatmulArgs a, int64_t B, hipStream_t st) {
     a.tiles_m = a.M / 256;
     a.tiles_n = a.S / (NW * 64);
     const dim3 grid(a.tiles_m * a.tiles_n, 1, (unsigned)B), block(NW * 128);
-    hipLaunchKernelGGL((matmul_kernel_pipe<BITS, NW>), grid, block, 0, st, a);
+    hipLaunchKernelGGL((matmul_kernel_pipe<BITS, SPARSE, NW>), grid, block, 0, st, a);
 }
 
 template <int BITS, bool SPARSE, int BM, int BN, int WM, int WN>
@@ -607,18 +703,19 @@ static void launch_tile(MatmulArgs a, int64_t B, hipStream_t st) {
 
 template <int BITS, bool SPARSE>
 static void launch(const MatmulArgs& a, int64_t B, hipStream_t st) {
-    // variant 0 = automatic.  Dense formats with tile-aligned shapes take the
-    // pipelined kernel: 256 x 128 tiles (two workgroups per CU) when there are
-    // enough of them to keep every CU at two, 256 x 256 tiles (one eight-wave
-    // workgroup per CU) for smaller grids.  Everything else: 128 x 256 tiles, and
-    // 128 x 128 for narrow outputs or few rows.
+    // variant 0 = automatic.  Tile-aligned shapes take the pipelined kernel:
+    // 256 x 128 tiles (two workgroups per CU) when there are enough of them to
+    // keep every CU at two, 256 x 256 tiles (one eight-wave workgroup per CU)
+    // for smaller grids and for the 16:32 format, whose decode needs more
+    // registers than the four-wave shape leaves.  Everything else: 128 x 256
+    // tiles, and 128 x 128 for narrow outputs or few rows.
     int variant = (int)tuning(TUNE_MM_VARIANT);
     const bool pipe2_ok = !SPARSE && a.M % 256 == 0 && a.S % 128 == 0;
-    const bool pipe4_ok = !SPARSE && a.M % 256 == 0 && a.S % 256 == 0;
+    const bool pipe4_ok = a.M % 256 == 0 && a.S % 256 == 0;
     if ((variant == 5 && !pipe2_ok) || (variant == 6 && !pipe4_ok)) variant = 0;
     if (variant == 0) {
         const int64_t tiles4 = (int64_t)(a.M / 256) * (a.S / 256) * B;
-        if (pipe4_ok && tiles4 <= 384) variant = 6;
+        if (pipe4_ok && (SPARSE || tiles4 <= 384)) variant = 6;
         else if (pipe2_ok) variant = 5;
         else if (a.M > 128 && a.S >= 256) variant = 3;
         else variant = 1;
@@ -627,10 +724,8 @@ static void launch(const MatmulArgs& a, int64_t B, hipStream_t st) {
     else if (variant == 2) launch_tile<BITS, SPARSE, 128, 256, 64, 128>(a, B, st);
     else if (variant == 3) launch_tile<BITS, SPARSE, 128, 256, 128, 64>(a, B, st);
     else if (variant == 4) launch_tile<BITS, SPARSE, 256, 256, 128, 64>(a, B, st);
-    else if constexpr (!SPARSE) {
-        if (variant == 6) launch_pipe<BITS, 4>(a, B, st);
-        else launch_pipe<BITS, 2>(a, B, st);
-    }
+    else if (variant == 6) launch_pipe<BITS, SPARSE, 4>(a, B, st);
+    else if constexpr (!SPARSE) launch_pipe<BITS, false, 2>(a, B, st);
 }
 
 }  // namespace i4
