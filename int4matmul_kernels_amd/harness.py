@@ -1,0 +1,217 @@
+"""Accuracy + timing harness of the quantized products on an MI355X.
+
+Plays the role of the reference's `kernel_test.py` (generation of test
+matrices `:160-236`, call convention `:254-259`, error metric `:261-262`, pass
+rule `:344-348`, timing loop `:290-309`, markdown table `:359-391`) through the
+drop-in `int4matmul` extension module, with three differences: matrices are
+packed on the device by the library's own packers, each row also reports the
+roofline figure of the kernel (GB/s for M = 1, TFLOP/s otherwise), and launches
+are additionally timed with HIP events.
+
+    python -m int4matmul_kernels_amd.harness                 # the standard configurations
+    python -m int4matmul_kernels_amd.harness --quick         # small shapes only
+    python -m int4matmul_kernels_amd.harness --config 4,5120,20480,2048,128,0
+
+A configuration is bits,K,S,M,group,sparse[,B].
+"""
+import argparse
+import time
+
+import torch
+
+import int4matmul_kernels_amd as pkg
+from int4matmul_kernels_amd import capi
+
+DEV = "cuda"
+
+# name, bits, K, S, M, group, sparse, B
+STANDARD = [
+    ("C1", 4, 1024, 1024, 1, 64, False, 1),
+    ("C2", 4, 5120, 20480, 1, 128, False, 1),
+    ("C2t", 4, 20480, 5120, 1, 128, False, 1),
+    ("C3", 4, 5120, 20480, 2048, 128, False, 1),
+    ("C3t", 4, 20480, 5120, 2048, 128, False, 1),
+    ("C3s", 4, 128, 128, 2048, 128, False, 1),
+    ("C4v", 4, 16384, 16384, 1, 64, True, 1),
+    ("C4m", 4, 5120, 20480, 2048, 64, True, 1),
+    ("C5v3", 3, 5120, 20480, 1, 128, False, 1),
+    ("C5m3", 3, 5120, 20480, 2048, 128, False, 1),
+    ("C5v2", 2, 5120, 20480, 1, 128, False, 1),
+    ("C5m2", 2, 5120, 20480, 2048, 128, False, 1),
+]
+QUICK = [
+    ("q4", 4, 1024, 1024, 1, 64, False, 1),
+    ("q4m", 4, 512, 512, 256, 128, False, 1),
+    ("q3", 3, 1024, 512, 70, 64, False, 2),
+    ("q2", 2, 512, 1024, 1, -1, False, 3),
+    ("q4s", 4, 1024, 512, 1, 64, True, 1),
+    ("q4sm", 4, 512, 512, 300, 64, True, 1),
+]
+
+
+def make_case(bits, K, S, M, group, sparse, B, seed=0):
+    """Synthetic problem: codes U{0..2^bits-1}, scales U(0.001, 0.02) (int4) or
+    U(0.004, 0.08), zeros U(0, 15) for int4 and the mid-code constant otherwise,
+    states N(0, 1); generated on the CPU with a fixed seed, packed on the device."""
+    gen = torch.Generator().manual_seed(seed)
+    codes = torch.randint(0, 1 << bits, (K, S), generator=gen, dtype=torch.int32).to(torch.uint8)
+    G = 1 if group < 0 else (K + group - 1) // group
+    lo, hi = (0.001, 0.02) if bits == 4 else (0.004, 0.08)
+    scales = (torch.rand((G, S), generator=gen) * (hi - lo) + lo).half()
+    if bits == 4:
+        zeros = (torch.rand((G, S), generator=gen) * 15.0).half()
+    else:
+        zeros = torch.full((G, S), ((1 << bits) - 1) / 2.0).half()
+    states = torch.randn((B, M, K), generator=gen).half()
+    codes_d = codes.to(DEV)
+    mask = None
+    if sparse:
+        # a random 16 of every 32 consecutive K per column
+        keys = torch.rand((S, K // 32, 32), generator=gen)
+        keep = torch.zeros((S, K // 32, 32), dtype=torch.uint8)
+        keep.scatter_(2, keys.argsort(dim=2)[:, :, :16], 1)
+        keep_d = keep.reshape(S, K).to(DEV)
+        matrix = torch.zeros((K // 16, S), dtype=torch.int32, device=DEV)
+        mask = torch.zeros((K // 32, S), dtype=torch.int32, device=DEV)
+        capi.sparse_pack(matrix, mask, codes_d.t().contiguous(), keep_d)
+    else:
+        matrix = torch.zeros((K * bits // 32, S), dtype=torch.int32, device=DEV)
+        capi.dense_pack(bits, matrix, codes_d)
+    return dict(bits=bits, K=K, S=S, M=M, B=B, group=group, matrix=matrix, mask=mask,
+                scales=scales.to(DEV), zeros=zeros.to(DEV), states=states.to(DEV))
+
+
+def reference_matrices(c):
+    """(fp16 weights exactly as the kernels' decode defines them, fp32 weights
+    dequantised in fp32) -- both through the library's unpack, then torch math"""
+    K, S, bits = c["K"], c["S"], c["bits"]
+    w16 = torch.empty((K, S), dtype=torch.float16, device=DEV)
+    capi.dequantize(bits, w16, c["matrix"], c["scales"], c["zeros"], c["group"], c["mask"])
+    codes = torch.empty((K, S), dtype=torch.uint8, device=DEV)
+    keep = torch.empty((K, S), dtype=torch.uint8, device=DEV)
+    capi.unpack(bits, codes, keep, c["matrix"], c["mask"])
+    g = K if c["group"] < 0 else c["group"]
+    rows = torch.arange(K, device=DEV) // g
+    s32, z32 = c["scales"].float()[rows], c["zeros"].float()[rows]
+    w32 = (codes.float() - z32) * s32 * keep.float()
+    return w16, w32
+
+
+def mean_rel_error(truth, cand):
+    """the reference's metric: nanmean(|(cand - truth) / truth|)"""
+    return ((cand.float() - truth) / truth).abs().nanmean().item()
+
+
+def algorithmic_bytes(c):
+    n = c["matrix"].numel() * 4 + c["scales"].numel() * 2 + c["zeros"].numel() * 2 + 2 * c["K"] + 2 * c["S"]
+    if c["mask"] is not None:
+        n += c["mask"].numel() * 4
+    return n
+
+
+def run_case(name, c, ext, repeats=100, trials=5):
+    B, M, K, S = c["B"], c["M"], c["K"], c["S"]
+    w16, w32 = reference_matrices(c)
+    truth = c["states"].float() @ w32
+
+    def quant():
+        outs = torch.zeros((B, M, S), dtype=torch.float16, device=DEV)
+        ext.quant_matmul(c["bits"], outs, c["matrix"], c["states"], c["scales"], c["zeros"], c["group"], c["mask"])
+        return outs
+
+    def fp16():
+        return c["states"] @ w16
+
+    err_q = mean_rel_error(truth, quant())
+    err_h = mean_rel_error(truth, fp16())
+    ok = err_q <= 0.1 or not (err_h == err_h)          # the reference's pass rule
+    out = {"name": name, "err_quant": err_q, "err_fp16": err_h, "ok": ok}
+    for label, fn in (("fp16", fp16), ("quant", quant)):
+        # reference-style wall clock: trials x repeats launches including the output allocation
+        fn()
+        torch.cuda.synchronize()
+        walls = []
+        for _ in range(trials):
+            t0 = time.time()
+            for _ in range(repeats):
+                fn()
+            torch.cuda.synchronize()
+            walls.append((time.time() - t0) / repeats)
+        out[label + "_wall_us"] = sum(walls) / len(walls) * 1e6
+    # kernel-only: HIP events around back-to-back launches into one output buffer
+    outs = torch.zeros((B, M, S), dtype=torch.float16, device=DEV)
+    call = lambda: ext.quant_matmul(c["bits"], outs, c["matrix"], c["states"], c["scales"], c["zeros"],
+                                    c["group"], c["mask"])
+    n = 200 if M == 1 else 20
+    for _ in range(5):
+        call()
+    torch.cuda.synchronize()
+    batches = []
+    for _ in range(5):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(n):
+            call()
+        e1.record()
+        torch.cuda.synchronize()
+        batches.append(e0.elapsed_time(e1) * 1e3 / n)
+    us = sorted(batches)[len(batches) // 2]
+    out["quant_event_us"] = us
+    if M * B == 1:
+        out["rate"] = "%.0f GB/s" % (algorithmic_bytes(c) / us / 1e3)
+    else:
+        out["rate"] = "%.1f TFLOP/s" % (2.0 * B * M * K * S / us / 1e6)
+    return out
+
+
+def table(rows, cases):
+    head = ["case", "B", "S", "N", "M", "", "weights", "states", "Time (us)", "kernel (us)", "rate", "mean rel err", ""]
+    body = []
+    for r, (name, bits, K, S, M, group, sparse, B) in zip(rows, cases):
+        sp = "16:32" if sparse else ""
+        body.append([name, B, S, K, M, sp, "fp16", "fp16", "%.2f" % r["fp16_wall_us"], "", "", "%.2e" % r["err_fp16"], ""])
+        body.append([name, B, S, K, M, sp, "int%d" % bits, "fp16", "%.2f" % r["quant_wall_us"],
+                     "%.2f" % r["quant_event_us"], r["rate"], "%.2e" % r["err_quant"], "ok" if r["ok"] else "FAIL"])
+    cols = list(zip(*([head] + [[str(x) for x in b] for b in body])))
+    widths = [max(len(x) for x in col) + 2 for col in cols]
+    lines = ["|" + "|".join(h.center(w) for h, w in zip(head, widths)) + "|",
+             "|" + "|".join(("-" * (w - 2)).center(w) for w in widths) + "|"]
+    for b in body:
+        lines.append("|" + "|".join(str(x).rjust(w - 1) + " " for x, w in zip(b, widths)) + "|")
+    return "\n".join(lines)
+
+
+def main(argv=None):
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("--quick", action="store_true", help="small shapes only")
+    ap.add_argument("--config", action="append", default=[], help="bits,K,S,M,group,sparse[,B]")
+    ap.add_argument("--repeats", type=int, default=100)
+    args = ap.parse_args(argv)
+    if not torch.cuda.is_available():
+        raise SystemExit("the harness needs a GPU")
+    ext = pkg.load_extension()
+    cases = QUICK if args.quick else STANDARD
+    if args.config:
+        cases = []
+        for i, spec in enumerate(args.config):
+            v = [int(x) for x in spec.split(",")]
+            cases.append(("u%d" % i, v[0], v[1], v[2], v[3], v[4], bool(v[5]), v[6] if len(v) > 6 else 1))
+    rows = []
+    for case in cases:
+        name, bits, K, S, M, group, sparse, B = case
+        c = make_case(bits, K, S, M, group, sparse, B)
+        rows.append(run_case(name, c, ext, repeats=args.repeats))
+        print("%-5s int%d K=%d S=%d M=%d B=%d g=%d %s: %.2f us, %s, mean rel err %.2e %s" % (
+            name, bits, K, S, M, B, group, "16:32" if sparse else "dense", rows[-1]["quant_event_us"],
+            rows[-1]["rate"], rows[-1]["err_quant"], "ok" if rows[-1]["ok"] else "FAIL"), flush=True)
+        del c
+        torch.cuda.empty_cache()
+    print()
+    print(table(rows, cases))
+    if not all(r["ok"] for r in rows):
+        raise SystemExit("a case exceeded the 10 % mean relative error gate")
+    return rows
+
+
+if __name__ == "__main__":
+    main()
