@@ -20,7 +20,7 @@ PKG = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG, "csrc")
 OBJ = os.path.join(PKG, "build")
 LIB = os.path.join(PKG, "libint4mm_hip.so")
-HIP_SOURCES = ["api.hip", "utils.hip", "matvec.hip", "matmul.hip"]
+HIP_SOURCES = ["api.hip", "utils.hip", "matvec.hip", "matmul.hip", "skinny.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 ARCH = "gfx950"
 

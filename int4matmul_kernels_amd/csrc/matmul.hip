@@ -744,6 +744,13 @@ extern "C" int int4mm_matmul(int bits, void* outs, const void* matrix, const voi
     if (((M + 127) / 128) * ((S + 127) / 128) > 0x7FFFFFFF / 2) return INT4MM_ERR_SHAPE;
     const int64_t g = shape->group_size < 0 ? ONE_GROUP : shape->group_size;
 
+    hipStream_t st = (hipStream_t)stream;
+    // 2 .. 32 rows in all (batches are contiguous, so they flatten): the HBM-bound few-row kernel
+    if (!sparse_mask && bits == 4 && B * M >= 2 && B * M <= 32 && !tuning(TUNE_NO_SKINNY) &&
+        skinny_int4((h16*)outs, (const uint32_t*)matrix, (const h16*)multiplier, (const h16*)scales,
+                    (const h16*)zeros, B * M, K, S, g, false, st))
+        return check_launch("matmul");
+
     MatmulArgs a;
     a.outs = (h16*)outs;
     a.matrix = (const uint32_t*)matrix;
@@ -757,7 +764,6 @@ extern "C" int int4mm_matmul(int bits, void* outs, const void* matrix, const voi
     a.group_units = (int)(g / 64 > 0x7FFFFFF ? 0x7FFFFFF : g / 64);
     a.tiles_m = a.tiles_n = 0;
 
-    hipStream_t st = (hipStream_t)stream;
     if (sparse_mask) launch<4, true>(a, B, st);
     else if (bits == 4) launch<4, false>(a, B, st);
     else if (bits == 3) launch<3, false>(a, B, st);

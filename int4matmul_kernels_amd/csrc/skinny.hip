@@ -1,0 +1,381 @@
+// Few-row product for gfx950: 2 .. 32 rows of states against a dense int4
+// weight matrix, HBM-bound like the matvec (every packed word is read once and
+// used for all rows).  The reference has no such path: it sends M >= 2 to its
+// 64-row matmul tiles (int4matmul.cpp:27) and M == 1 with B > 1 to one matvec
+// per batch element, re-reading the weights each time (matvec_kernel.cu:346).
+//
+// The rows are multiplied on the matrix core: v_mfma_f32_16x16x32_f16 takes 16
+// rows of states as its 16 x 32 operand (rows >= R are zero; 17 .. 32 rows take
+// two such tiles) and, as its 32 x 16 operand, 8 consecutive k of one column per
+// lane -- which is exactly one packed int4 word; the four lane groups of a wave
+// hold the four packed rows of a 32-row block.  A word becomes that operand without converting a single code:
+// mask-and-OR of the word (and of the word shifted by 8) gives the half2 pairs
+// {1024 + q0, 1024 + q4}, {64 + q1, 64 + q5}, {1024 + q2, 1024 + q6}, {64 + q3,
+// 64 + q7}; the states are stored to LDS in the same k order 0,4,1,5,2,6,3,7.
+// The offsets are removed once per quantisation group in fp32 together with
+// scale and zero:
+//     y[m, n] += s[n] * (acc[m, n] - sum_k off_k x[m, k] - z[n] * sum_k x[m, k])
+// which is the exact value of sum_k x (q - z) s (the per-weight fp16 roundings of
+// the reference's decode are not reproduced, as in the matvec).
+//
+// A workgroup owns a strip of 16 * CW columns (lane j of a wave holds the words
+// of CW adjacent columns: CW * 64 contiguous bytes per packed row and wave) and
+// its W waves split K; each wave stages the states of its own K range through
+// a private LDS buffer, 64 k at a time, and the partial tiles are summed
+// through LDS at the end -- no exchange between workgroups.
+#include "common.h"
+
+#include <type_traits>
+
+namespace i4 {
+
+struct SkinnyArgs {
+    h16* outs;
+    const uint32_t* matrix;
+    const h16* x;
+    const h16* scales;
+    const h16* zeros;
+    int R, K, S;
+    int group_units;        // group size / 64
+    int units_per_wave;
+    int accumulate;         // 1: outs = fp16(fp32(outs) + product) (matvec semantics); 0: overwrite
+};
+
+constexpr int SK_PITCH = 144;                   // bytes between rows of a staged unit (128 + 16: conflict-free)
+constexpr int SK_XBUF = 32 * SK_PITCH;          // one staged unit: 32 rows x 64 k
+constexpr int SK_WAVE_LDS = 2 * SK_XBUF + 256;  // two unit buffers + the group sums of 32 rows
+
+template <int CW> struct Words;
+template <> struct Words<4> { typedef u32x4 type; };
+template <> struct Words<2> { typedef u32x2 type; };
+template <> struct Words<1> { typedef uint32_t type; };
+
+template <int CW>
+__device__ __forceinline__ uint32_t word_of(const typename Words<CW>::type& v, int c) {
+    if constexpr (CW == 1) return v;
+    else return v[c];
+}
+
+// A 32-bit constant kept in a VGPR: VOP3 encodings on this target cannot carry two
+// different literals, so v_and_or_b32 is only selected when mask and magic are
+// registers.  The expression itself stays visible to the compiler, which has to
+// track the VALU -> MFMA operand hazards.
+__device__ __forceinline__ uint32_t vgpr_const(uint32_t literal) {
+    uint32_t r;
+    asm("v_mov_b32 %0, %1" : "=v"(r) : "s"(literal));
+    return r;
+}
+
+// k order of the 8 halves of an operand chunk
+__device__ constexpr int SK_ORDER[8] = {0, 4, 1, 5, 2, 6, 3, 7};
+
+// packed word -> MFMA operand {1024 + q0, 1024 + q4, 64 + q1, 64 + q5, 1024 + q2, ...}
+__device__ __forceinline__ h16x8 magic_operand_int4(uint32_t u, uint32_t m0, uint32_t m1, uint32_t g0, uint32_t g1) {
+    const uint32_t u8 = u >> 8;
+    const u32x4 r = {(u & m0) | g0, (u & m1) | g1, (u8 & m0) | g0, (u8 & m1) | g1};
+    return bitcast<h16x8>(r);
+}
+
+__device__ __forceinline__ h16x8 exact_operand_int4(uint32_t u, h16 sc, h16 ze) {
+    h16x8 r;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) r[e] = dequant_code<4>((u >> (4 * SK_ORDER[e])) & 15u, sc, ze);
+    return r;
+}
+
+// CW: columns per lane; RT: row groups of 8 that can hold real rows (R <= 8 RT);
+// MT: 16-row MFMA tiles; PF: units of packed weights in flight per wave
+template <int CW, int RT>
+__global__ __launch_bounds__(512) void skinny_kernel(SkinnyArgs a) {
+    constexpr int PF = 4, MT = RT == 4 ? 2 : 1;
+    constexpr int PFX = RT == 4 ? 2 : 4;            // units of states in flight per wave
+    constexpr int STRIP = 16 * CW;
+    extern __shared__ __attribute__((aligned(16))) char lds[];
+    typedef typename Words<CW>::type words_t;
+    const int t = threadIdx.x, lane = t & 63, nwaves = blockDim.x >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);   // scalar: the unit loop runs on SGPRs
+    const int j = lane & 15, h = lane >> 4;
+    const int col0 = blockIdx.x * STRIP + CW * j;              // first of this lane's CW columns
+    const int units = a.K / 64;
+    const int u0 = wave * a.units_per_wave, u1 = min(units, u0 + a.units_per_wave);
+
+    // The strip's scales and zeros ([groups][STRIP] halves each) are copied to LDS
+    // once: the loop then never waits on a global load other than its prefetched
+    // weights and states.  Exponent-mode scales (negative or NaN) anywhere in the
+    // strip switch the whole workgroup to the exact per-weight decode.  (The copy
+    // runs after the first loads have been issued, under their latency.)
+    const int groups = (units + a.group_units - 1) / a.group_units;
+    uint32_t* sz = reinterpret_cast<uint32_t*>(lds + nwaves * SK_WAVE_LDS + 16);      // scales, then zeros
+    auto scan_scales = [&]() -> bool {
+        int* flag = reinterpret_cast<int*>(lds + nwaves * SK_WAVE_LDS);
+        if (t == 0) *flag = 0;
+        __syncthreads();
+        bool bad = false;
+        const int n = groups * (STRIP / 2);
+        for (int i = t; i < n; i += blockDim.x) {
+            const int g = i / (STRIP / 2), c = i % (STRIP / 2);
+            const int64_t at = (int64_t)g * a.S + blockIdx.x * STRIP + 2 * c;
+            const uint32_t two = *reinterpret_cast<const uint32_t*>(a.scales + at);
+            bad |= !(as_h2(two).x >= (h16)0.0f) || !(as_h2(two).y >= (h16)0.0f);
+            sz[i] = two;
+            sz[n + i] = *reinterpret_cast<const uint32_t*>(a.zeros + at);
+        }
+        if (__builtin_amdgcn_ballot_w64(bad) != 0 && lane == 0) *flag = 1;
+        __syncthreads();
+        return *flag != 0;
+    };
+    bool general = false;
+
+    char* my = lds + wave * SK_WAVE_LDS;
+    float* sums = reinterpret_cast<float*>(my + 2 * SK_XBUF);   // [0..31] sum x, [32..63] sum off x
+
+    // accumulators: acc = raw products of the current group, y = finished groups
+    // (register e of tile mt is row 16 mt + 4 h + e, column j)
+    f32x4 acc[CW][MT], y[CW][MT];
+#pragma unroll
+    for (int c = 0; c < CW; ++c)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) { acc[c][mt] = f32x4{0.f, 0.f, 0.f, 0.f}; y[c][mt] = f32x4{0.f, 0.f, 0.f, 0.f}; }
+
+    if (u0 >= u1) general = scan_scales();          // idle waves still take part in its barriers
+    if (u0 < u1) {
+        // ---- loaders
+        // weights of unit u: packed rows 8u + 4 blk + h, blk = 0, 1, CW words each
+        const uint32_t* wbase = a.matrix + (int64_t)h * a.S + col0;
+        const int64_t wrow4 = (int64_t)4 * a.S;
+        auto load_w = [&](words_t w[2], int u) {
+            const uint32_t* p = wbase + (int64_t)u * 8 * a.S;
+#pragma unroll
+            for (int i = 0; i < 2; ++i) w[i] = __builtin_nontemporal_load(reinterpret_cast<const words_t*>(p + i * wrow4));
+        };
+        // states of unit u (8 RT rows x 128 bytes): 8 / RT lanes per row, RT 16-byte chunks
+        // each; the rows of the LDS buffers beyond 8 RT stay zero
+        constexpr int LPR = 8 / RT;                                   // lanes per row
+        const int xm = lane / LPR, xpart = lane % LPR;
+        const bool xreal = xm < a.R;
+        const h16* xsrc = a.x + (int64_t)min(xm, a.R - 1) * a.K + xpart * (8 * RT);
+        auto load_x = [&](u32x4 xr[RT], int u) {
+#pragma unroll
+            for (int i = 0; i < RT; ++i)
+                xr[i] = xreal ? *reinterpret_cast<const u32x4*>(xsrc + u * 64 + i * 8) : u32x4{0, 0, 0, 0};
+        };
+        // store a loaded unit to LDS buffer p and return its per-row sums (all lanes of a row get them)
+        auto stage_x = [&](const u32x4 xr[RT], int p, float& sx, float& so) {
+            const uint32_t ONES = 0x3C003C00u, OFF_A = 0x64006400u, OFF_B = 0x54005400u;   // 1, 1024, 64
+            sx = 0.f; so = 0.f;
+#pragma unroll
+            for (int i = 0; i < RT; ++i) {
+                const u32x4 v = xr[i];
+                // k order 0,4,1,5,2,6,3,7 inside the chunk, as the operand decode produces it
+                const u32x4 q = {__builtin_amdgcn_perm(v[2], v[0], 0x05040100u), __builtin_amdgcn_perm(v[2], v[0], 0x07060302u),
+                                 __builtin_amdgcn_perm(v[3], v[1], 0x05040100u), __builtin_amdgcn_perm(v[3], v[1], 0x07060302u)};
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    sx = dot2(q[e], ONES, sx);
+                    so = dot2(q[e], (e & 1) ? OFF_B : OFF_A, so);
+                }
+                *reinterpret_cast<u32x4*>(my + p * SK_XBUF + xm * SK_PITCH + (xpart * RT + i) * 16) = q;
+            }
+            // the other lanes of the row: lane ^ 1, lane ^ 2, lane ^ 4 as far as the row extends
+            sx += dpp_f32<0xB1>(sx);
+            so += dpp_f32<0xB1>(so);
+            if constexpr (LPR >= 4) { sx += dpp_f32<0x4E>(sx); so += dpp_f32<0x4E>(so); }
+            if constexpr (LPR >= 8) { sx += dpp_f32<0x141>(sx); so += dpp_f32<0x141>(so); }
+        };
+        // rows that never receive states must read as zero
+        for (int i = lane; i < 2 * SK_XBUF / 16; i += 64) *reinterpret_cast<u32x4*>(my + i * 16) = u32x4{0, 0, 0, 0};
+
+        words_t w[PF][2];
+        u32x4 xr[PFX][RT];
+        const uint32_t m0 = vgpr_const(0x000F000Fu), m1 = vgpr_const(0x00F000F0u);
+        const uint32_t g0 = vgpr_const(0x64006400u), g1 = vgpr_const(0x54005400u);
+        float gS = 0.f, gO = 0.f;           // sums of the current group so far (row lane / 2)
+        float nS, nO;                       // sums of the unit staged last (the next to be multiplied)
+        // scale / zero of the lane's CW columns for group gi, from the LDS copy
+        h16 sc[CW], ze[CW];
+#pragma unroll
+        for (int c = 0; c < CW; ++c) { sc[c] = (h16)0.f; ze[c] = (h16)0.f; }
+        auto load_sz = [&](int gi) {
+            const h16* ps = reinterpret_cast<const h16*>(sz) + gi * STRIP + CW * j;
+            const h16* pz = ps + groups * STRIP;
+            if constexpr (CW == 4) {
+                const u32x2 s2 = *reinterpret_cast<const u32x2*>(ps), z2 = *reinterpret_cast<const u32x2*>(pz);
+                sc[0] = as_h2(s2.x).x; sc[1] = as_h2(s2.x).y; sc[2] = as_h2(s2.y).x; sc[3] = as_h2(s2.y).y;
+                ze[0] = as_h2(z2.x).x; ze[1] = as_h2(z2.x).y; ze[2] = as_h2(z2.y).x; ze[3] = as_h2(z2.y).y;
+            } else if constexpr (CW == 2) {
+                const uint32_t s1 = *reinterpret_cast<const uint32_t*>(ps), z1 = *reinterpret_cast<const uint32_t*>(pz);
+                sc[0] = as_h2(s1).x; sc[1] = as_h2(s1).y; ze[0] = as_h2(z1).x; ze[1] = as_h2(z1).y;
+            } else {
+                sc[0] = ps[0]; ze[0] = pz[0];
+            }
+        };
+
+#pragma unroll
+        for (int f = 0; f < PF; ++f) load_w(w[f], min(u0 + f, u1 - 1));
+        load_x(xr[0], u0);
+        general = scan_scales();
+        stage_x(xr[0], 0, nS, nO);
+        // set f holds unit u0 + f (f >= 1) and, for f = 0, unit u0 + PFX
+#pragma unroll
+        for (int f = 1; f <= PFX; ++f) load_x(xr[f % PFX], min(u0 + f, u1 - 1));
+
+        // p: parity of the LDS buffer that holds unit u; xn: the register set with the states of unit u + 1.
+        // The decode mode is a compile-time tag: one loop body per mode, no branches inside.
+        auto step = [&](auto mode, int u, int p, words_t w[2], u32x4 xn[RT]) {
+            constexpr bool general = decltype(mode)::value;
+            if constexpr (general) {
+                if (u == u0 || u % a.group_units == 0) load_sz(u / a.group_units);
+            }
+            gS += nS; gO += nO;
+            // 2 blocks of 32 k: lane group h multiplies chunk h (8 k) of the block
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                h16x8 xa[MT];
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt)
+                    xa[mt] = *reinterpret_cast<const h16x8*>(my + p * SK_XBUF + (j + 16 * mt) * SK_PITCH + (i * 4 + h) * 16);
+#pragma unroll
+                for (int c = 0; c < CW; ++c) {
+                    const uint32_t word = word_of<CW>(w[i], c);
+                    const h16x8 wb = general ? exact_operand_int4(word, sc[c], ze[c])
+                                             : magic_operand_int4(word, m0, m1, g0, g1);
+#pragma unroll
+                    for (int mt = 0; mt < MT; ++mt)
+                        acc[c][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[mt], wb, acc[c][mt], 0, 0, 0);
+                }
+            }
+            // refill this register set PF units ahead; move the next unit's states to LDS
+            load_w(w, min(u + PF, u1 - 1));
+            stage_x(xn, p ^ 1, nS, nO);
+            load_x(xn, min(u + 1 + PFX, u1 - 1));
+            // group complete (or this wave's range ends): fold it into y
+            if ((u + 1) % a.group_units == 0 || u + 1 == u1) {
+                if (xpart == 0) { sums[xm] = gS; sums[32 + xm] = gO; }
+                if constexpr (!general) load_sz(u / a.group_units);
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) {
+                    const f32x4 s4 = *reinterpret_cast<const f32x4*>(&sums[16 * mt + 4 * h]);
+                    const f32x4 o4 = *reinterpret_cast<const f32x4*>(&sums[32 + 16 * mt + 4 * h]);
+#pragma unroll
+                    for (int c = 0; c < CW; ++c) {
+                        const float sf = general ? 1.f : (float)sc[c];
+                        const float z = general ? 0.f : (float)ze[c];
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const float off = general ? 0.f : o4[e] + z * s4[e];
+                            y[c][mt][e] += sf * (acc[c][mt][e] - off);
+                        }
+                        acc[c][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+                    }
+                }
+                gS = 0.f; gO = 0.f;
+            }
+        };
+        auto run = [&](auto mode) {
+            for (int u = u0; u < u1; u += PF) {
+#pragma unroll
+                for (int f = 0; f < PF; ++f) {
+                    if (f > 0 && u + f >= u1) break;
+                    step(mode, u + f, f & 1, w[f], xr[(f + 1) % PFX]);
+                }
+            }
+        };
+        if (general) run(std::integral_constant<bool, true>{});
+        else run(std::integral_constant<bool, false>{});
+    }
+
+    // ---- sum the waves' partial tiles through LDS (tile: [16 MT rows][16 CW columns] fp32)
+    __syncthreads();
+    constexpr int TILE = MT * 16 * STRIP;
+    float* red = reinterpret_cast<float*>(lds);
+    auto tile_at = [&](float* base, int mt, int e) { return base + ((mt * 16 + 4 * h + e) * 16 + j) * CW; };
+    for (int s = nwaves >> 1; s >= 1; s >>= 1) {
+        if (wave >= s && wave < 2 * s) {
+            float* dst = red + (wave - s) * TILE;
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+#pragma unroll
+                    for (int c = 0; c < CW; ++c) tile_at(dst, mt, e)[c] = y[c][mt][e];
+        }
+        __syncthreads();
+        if (wave < s) {
+            float* src = red + wave * TILE;
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+#pragma unroll
+                    for (int c = 0; c < CW; ++c) y[c][mt][e] += tile_at(src, mt, e)[c];
+        }
+        __syncthreads();
+    }
+    if (wave == 0) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int m = mt * 16 + 4 * h + e;
+                if (m < a.R) {
+                    h16* o = a.outs + (int64_t)m * a.S + col0;
+#pragma unroll
+                    for (int c = 0; c < CW; ++c) {
+                        float v = y[c][mt][e];
+                        if (a.accumulate) v += (float)o[c];
+                        o[c] = (h16)v;
+                    }
+                }
+            }
+    }
+}
+
+template <int CW>
+static bool launch_skinny(const SkinnyArgs& a, int waves, hipStream_t st) {
+    const int strips = a.S / (16 * CW);
+    const int rt = (a.R + 7) / 8;
+    const int groups = (a.K / 64 + a.group_units - 1) / a.group_units;
+    size_t lds = (size_t)waves * SK_WAVE_LDS + 16 + (size_t)groups * 16 * CW * 4;
+    const size_t red = (size_t)(waves / 2) * (rt <= 2 ? 1 : 2) * 16 * 16 * CW * 4;
+    if (red > lds) lds = red;
+    if (lds > 150 * 1024) return false;
+    const dim3 grid(strips), block(waves * 64);
+    auto go = [&](auto kernel) {
+        // more than 64 KB of dynamic LDS has to be requested per kernel
+        hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            150 * 1024);
+        hipLaunchKernelGGL(kernel, grid, block, lds, st, a);
+    };
+    if (rt <= 1) go(skinny_kernel<CW, 1>);
+    else if (rt <= 2) go(skinny_kernel<CW, 2>);
+    else go(skinny_kernel<CW, 4>);
+    return true;
+}
+
+// Product of R <= 32 rows with a dense int4 matrix.  Returns false when the shape
+// is not one this kernel takes (the caller then uses the general kernels).
+bool skinny_int4(h16* outs, const uint32_t* matrix, const h16* x, const h16* scales, const h16* zeros,
+                 int64_t R, int64_t K, int64_t S, int64_t group_size, bool accumulate, hipStream_t st) {
+    if (R < 2 || R > 32 || S % 16 != 0 || K % 64 != 0 || K > (1 << 30) || S > (1 << 28)) return false;
+    SkinnyArgs a;
+    a.outs = outs; a.matrix = matrix; a.x = x; a.scales = scales; a.zeros = zeros;
+    a.R = (int)R; a.K = (int)K; a.S = (int)S;
+    const int64_t gu = group_size / 64;
+    a.group_units = (int)(gu > 0x7FFFFFF ? 0x7FFFFFF : gu);
+    a.accumulate = accumulate ? 1 : 0;
+    // widest strips (16, 32 or 64 columns) that still give at least 256 workgroups;
+    // four waves split K when there are that many workgroups (three of them fit a
+    // CU), eight otherwise
+    int cw = 4;
+    while (cw > 1 && (S % (16 * cw) != 0 || S / (16 * cw) < 256)) cw >>= 1;
+    const int units = (int)(K / 64);
+    int waves = (int)tuning(TUNE_MV_WAVES);
+    if (waves != 2 && waves != 4 && waves != 8) waves = S / (16 * cw) >= 256 ? 4 : 8;
+    while (waves > 1 && units < 2 * waves) waves >>= 1;
+    a.units_per_wave = (units + waves - 1) / waves;
+    if (cw == 4) return launch_skinny<4>(a, waves, st);
+    if (cw == 2) return launch_skinny<2>(a, waves, st);
+    return launch_skinny<1>(a, waves, st);
+}
+
+}  // namespace i4
