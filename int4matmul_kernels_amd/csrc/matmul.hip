@@ -670,9 +670,9 @@ __device__ __forceinline__ void pipe_tile(const MatmulArgs& a, const int m0, con
         }
 }
 
-template <int BITS, bool SPARSE, int NW>
+template <int BITS, bool SPARSE, int NW, int TM>
 __global__ __launch_bounds__(NW * 128, NW == 2 ? 2 : 1) void matmul_kernel_pipe(MatmulArgs a) {
-    constexpr int BM = 256, BN = NW * 64;
+    constexpr int BM = TM * 64, BN = NW * 64;
     __shared__ __attribute__((aligned(16))) h16 As[P_STAGES * BM * PK];
     __shared__ __attribute__((aligned(16))) h16 Bs[P_STAGES * PK * BN];
     __shared__ __attribute__((aligned(16))) uint32_t Lut[SPARSE ? SPARSE_LUT_WORDS : 4];
@@ -681,16 +681,16 @@ __global__ __launch_bounds__(NW * 128, NW == 2 ? 2 : 1) void matmul_kernel_pipe(
     if (total % 8 == 0) bid = (bid % 8) * (total / 8) + bid / 8;     // XCD-aware renumbering
     const int tile_m = bid % a.tiles_m, tile_n = bid / a.tiles_m;
     const int64_t boff = blockIdx.z;
-    pipe_tile<BITS, SPARSE, 4, NW>(a, tile_m * BM, tile_n * BN, a.x + boff * a.M * (int64_t)a.K,
+    pipe_tile<BITS, SPARSE, TM, NW>(a, tile_m * BM, tile_n * BN, a.x + boff * a.M * (int64_t)a.K,
                                    a.outs + boff * a.M * (int64_t)a.S, As, Bs, Lut);
 }
 
-template <int BITS, bool SPARSE, int NW>
+template <int BITS, bool SPARSE, int NW, int TM = 4>
 static void launch_pipe(MatmulArgs a, int64_t B, hipStream_t st) {
-    a.tiles_m = a.M / 256;
+    a.tiles_m = a.M / (TM * 64);
     a.tiles_n = a.S / (NW * 64);
     const dim3 grid(a.tiles_m * a.tiles_n, 1, (unsigned)B), block(NW * 128);
-    hipLaunchKernelGGL((matmul_kernel_pipe<BITS, SPARSE, NW>), grid, block, 0, st, a);
+    hipLaunchKernelGGL((matmul_kernel_pipe<BITS, SPARSE, NW, TM>), grid, block, 0, st, a);
 }
 
 template <int BITS, bool SPARSE, int BM, int BN, int WM, int WN>
@@ -703,21 +703,25 @@ static void launch_tile(MatmulArgs a, int64_t B, hipStream_t st) {
 
 template <int BITS, bool SPARSE>
 static void launch(const MatmulArgs& a, int64_t B, hipStream_t st) {
-    // variant 0 = automatic.  Tile-aligned shapes take the pipelined kernel:
-    // 256 x 128 tiles (two workgroups per CU) when there are enough of them to
-    // keep every CU at two, 256 x 256 tiles (one eight-wave workgroup per CU)
-    // for smaller grids and for the 16:32 format, whose decode needs more
-    // registers than the four-wave shape leaves.  Everything else: 128 x 256
-    // tiles, and 128 x 128 for narrow outputs or few rows.
+    // variant 0 = automatic.  Tile-aligned shapes take the pipelined kernel, as
+    // 256 x 256 tiles (one eight-wave workgroup per CU) or 256 x 128 tiles (two
+    // four-wave workgroups per CU).  Measured on MI355X: the large tiles win when
+    // they fill their last round of 256 well; the small ones when fewer than half
+    // of the CUs would get a large tile, or when the large tiles' last round is at
+    // most half full.  The 16:32 format always takes the large tiles (its decode
+    // needs more registers than the four-wave shape leaves).  Everything else:
+    // 128 x 256 tiles, and 128 x 128 for narrow outputs or few rows.
     int variant = (int)tuning(TUNE_MM_VARIANT);
     const bool pipe2_ok = !SPARSE && a.M % 256 == 0 && a.S % 128 == 0;
     const bool pipe4_ok = a.M % 256 == 0 && a.S % 256 == 0;
     if ((variant == 5 && !pipe2_ok) || (variant == 6 && !pipe4_ok)) variant = 0;
     if (variant == 0) {
         const int64_t tiles4 = (int64_t)(a.M / 256) * (a.S / 256) * B;
-        if (pipe4_ok && (SPARSE || tiles4 <= 384)) variant = 6;
+        const int64_t last = tiles4 % 256;
+        const bool small_better = tiles4 < 128 || (tiles4 > 256 && last > 0 && last <= 128);
+        if (pipe4_ok && (SPARSE || !pipe2_ok || !small_better)) variant = 6;
         else if (pipe2_ok) variant = 5;
-        else if (a.M > 128 && a.S >= 256) variant = 3;
+        else if (a.M > 512 && a.S >= 256) variant = 3;
         else variant = 1;
     }
     if (variant == 1) launch_tile<BITS, SPARSE, 128, 128, 64, 64>(a, B, st);
