@@ -386,7 +386,8 @@ __device__ __forceinline__ void pipe_tile(const MatmulArgs& a, const int m0, con
     // states stage: row m at m * 64 bytes, 16-byte chunk c of the row stored at
     // c ^ ((m >> 2) & 3): sixteen consecutive rows read the same logical chunk
     // from sixteen different bank groups.  Thread t moves chunk t % 4 of rows
-    // t / 4 + A_ROWS * i through registers.  The tile lies inside the matrix
+    // t / 4 + A_ROWS * i through registers (rows >= M re-read row M - 1 and are
+    // dropped at the store).  The tile's columns lie inside the matrix
     // (launcher's duty).
     struct AStage { u32x4 v[A_LOADS]; };
     const int a_row = t >> 2, a_chunk = t & 3;
@@ -395,7 +396,8 @@ __device__ __forceinline__ void pipe_tile(const MatmulArgs& a, const int m0, con
     const char* const a_tile = reinterpret_cast<const char*>(x + (int64_t)m0 * a.K);
     uint32_t a_off[A_LOADS];
 #pragma unroll
-    for (int i = 0; i < A_LOADS; ++i) a_off[i] = (uint32_t)(((a_row + A_ROWS * i) * a.K + a_chunk * 8) * 2);
+    for (int i = 0; i < A_LOADS; ++i)
+        a_off[i] = (uint32_t)((min(a_row + A_ROWS * i, a.M - 1 - m0) * a.K + a_chunk * 8) * 2);
     const int a_dst = a_row * PK + ((a_chunk ^ ((a_row >> 2) & 3)) << 3);       // halves; rows + A_ROWS: same swizzle
     auto load_a = [&](AStage& r, const char* base) {
 #pragma unroll
@@ -665,7 +667,7 @@ __device__ __forceinline__ void pipe_tile(const MatmulArgs& a, const int m0, con
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int row = m0 + wm0 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-                outs[(int64_t)row * a.S + col] = (h16)acc[i][j][r];
+                if (row < a.M) outs[(int64_t)row * a.S + col] = (h16)acc[i][j][r];
             }
         }
 }
@@ -687,7 +689,7 @@ __global__ __launch_bounds__(NW * 128, NW == 2 ? 2 : 1) void matmul_kernel_pipe(
 
 template <int BITS, bool SPARSE, int NW, int TM = 4>
 static void launch_pipe(MatmulArgs a, int64_t B, hipStream_t st) {
-    a.tiles_m = a.M / (TM * 64);
+    a.tiles_m = (a.M + TM * 64 - 1) / (TM * 64);
     a.tiles_n = a.S / (NW * 64);
     const dim3 grid(a.tiles_m * a.tiles_n, 1, (unsigned)B), block(NW * 128);
     hipLaunchKernelGGL((matmul_kernel_pipe<BITS, SPARSE, NW, TM>), grid, block, 0, st, a);
@@ -712,11 +714,14 @@ static void launch(const MatmulArgs& a, int64_t B, hipStream_t st) {
     // needs more registers than the four-wave shape leaves).  Everything else:
     // 128 x 256 tiles, and 128 x 128 for narrow outputs or few rows.
     int variant = (int)tuning(TUNE_MM_VARIANT);
-    const bool pipe2_ok = !SPARSE && a.M % 256 == 0 && a.S % 128 == 0;
-    const bool pipe4_ok = a.M % 256 == 0 && a.S % 256 == 0;
+    // (M is padded to whole tiles; worth it while the padding stays below an eighth of M)
+    const int64_t m_pad = (a.M + 255) / 256 * 256;
+    const bool m_ok = (m_pad - a.M) * 8 <= a.M;
+    const bool pipe2_ok = !SPARSE && m_ok && a.S % 128 == 0;
+    const bool pipe4_ok = m_ok && a.S % 256 == 0;
     if ((variant == 5 && !pipe2_ok) || (variant == 6 && !pipe4_ok)) variant = 0;
     if (variant == 0) {
-        const int64_t tiles4 = (int64_t)(a.M / 256) * (a.S / 256) * B;
+        const int64_t tiles4 = m_pad / 256 * (a.S / 256) * B;
         const int64_t last = tiles4 % 256;
         const bool small_better = tiles4 < 128 || (tiles4 > 256 && last > 0 && last <= 128);
         if (pipe4_ok && (SPARSE || !pipe2_ok || !small_better)) variant = 6;

@@ -89,7 +89,7 @@ def test_degenerate_known_answer(H, bits, sparse, K):
 
 # ------------------------------------------------------------------- matmul
 @pytest.mark.parametrize("bits,sparse", FORMATS)
-@pytest.mark.parametrize("M,K,S,g", [(2048, 128, 128, 128), (70, 256, 192, 64), (1, 512, 64, 128),
+@pytest.mark.parametrize("M,K,S,g", [(2048, 128, 128, 128), (70, 256, 192, 64), (1, 512, 64, 128), (500, 192, 256, 64),
                                      (257, 1024, 320, -1)])
 def test_matmul_parity(H, bits, sparse, M, K, S, g):
     p = _problem(bits, sparse, K=K, S=S, M=M, group_size=g, seed=M)
