@@ -25,6 +25,7 @@
 // through LDS at the end -- no exchange between workgroups.
 #include "common.h"
 
+#include <atomic>
 #include <type_traits>
 
 namespace i4 {
@@ -340,15 +341,22 @@ static bool launch_skinny(const SkinnyArgs& a, int waves, hipStream_t st) {
     if (red > lds) lds = red;
     if (lds > 150 * 1024) return false;
     const dim3 grid(strips), block(waves * 64);
-    auto go = [&](auto kernel) {
-        // more than 64 KB of dynamic LDS has to be requested per kernel
-        hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                            150 * 1024);
+    auto go = [&](auto kernel, int slot) {
+        // more than 64 KB of dynamic LDS has to be requested once per kernel and device
+        static std::atomic<uint64_t> done[3];
+        int dev = 0;
+        hipGetDevice(&dev);
+        const uint64_t bit = 1ull << (dev & 63);
+        if (!(done[slot].load(std::memory_order_relaxed) & bit)) {
+            hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                150 * 1024);
+            done[slot].fetch_or(bit, std::memory_order_relaxed);
+        }
         hipLaunchKernelGGL(kernel, grid, block, lds, st, a);
     };
-    if (rt <= 1) go(skinny_kernel<CW, 1>);
-    else if (rt <= 2) go(skinny_kernel<CW, 2>);
-    else go(skinny_kernel<CW, 4>);
+    if (rt <= 1) go(skinny_kernel<CW, 1>, 0);
+    else if (rt <= 2) go(skinny_kernel<CW, 2>, 1);
+    else go(skinny_kernel<CW, 4>, 2);
     return true;
 }
 
