@@ -371,11 +371,14 @@ bool skinny_int4(h16* outs, const uint32_t* matrix, const h16* x, const h16* sca
     const int64_t gu = group_size / 64;
     a.group_units = (int)(gu > 0x7FFFFFF ? 0x7FFFFFF : gu);
     a.accumulate = accumulate ? 1 : 0;
-    // widest strips (16, 32 or 64 columns) that still give at least 256 workgroups;
-    // four waves split K when there are that many workgroups (three of them fit a
-    // CU), eight otherwise
-    int cw = 4;
-    while (cw > 1 && (S % (16 * cw) != 0 || S / (16 * cw) < 256)) cw >>= 1;
+    // widest strips (64, 32 or 16 columns) that still give at least 256 workgroups,
+    // else at least 128 (narrow strips use half a cache line per packed row);
+    // four waves split K when there are 256 workgroups (three of them fit a CU),
+    // eight otherwise
+    int cw = 1;
+    const int prefer[4][2] = {{4, 256}, {2, 256}, {4, 128}, {2, 128}};       // {columns per lane, workgroups}
+    for (const auto& c : prefer)
+        if (S % (16 * c[0]) == 0 && S / (16 * c[0]) >= c[1]) { cw = c[0]; break; }
     const int units = (int)(K / 64);
     int waves = (int)tuning(TUNE_MV_WAVES);
     if (waves != 2 && waves != 4 && waves != 8) waves = S / (16 * cw) >= 256 ? 4 : 8;
