@@ -716,7 +716,8 @@ static void launch(const MatmulArgs& a, int64_t B, hipStream_t st) {
     int variant = (int)tuning(TUNE_MM_VARIANT);
     // (M is padded to whole tiles; worth it while the padding stays below an eighth of M)
     const int64_t m_pad = (a.M + 255) / 256 * 256;
-    const bool m_ok = (m_pad - a.M) * 8 <= a.M;
+    // (the kernel's per-lane byte offsets are 32-bit: 256 rows of states, 4 packed rows of weights)
+    const bool m_ok = (m_pad - a.M) * 8 <= a.M && a.K <= (1 << 22) && a.S <= (1 << 27);
     const bool pipe2_ok = !SPARSE && m_ok && a.S % 128 == 0;
     const bool pipe4_ok = m_ok && a.S % 256 == 0;
     if ((variant == 5 && !pipe2_ok) || (variant == 6 && !pipe4_ok)) variant = 0;
@@ -755,8 +756,8 @@ extern "C" int int4mm_matmul(int bits, void* outs, const void* matrix, const voi
 
     hipStream_t st = (hipStream_t)stream;
     // 2 .. 32 rows in all (batches are contiguous, so they flatten): the HBM-bound few-row kernel
-    if (!sparse_mask && bits == 4 && B * M >= 2 && B * M <= 32 && !tuning(TUNE_NO_SKINNY) &&
-        skinny_int4((h16*)outs, (const uint32_t*)matrix, (const h16*)multiplier, (const h16*)scales,
+    if (!sparse_mask && B * M >= 2 && B * M <= 32 && !tuning(TUNE_NO_SKINNY) &&
+        skinny_dense(bits, (h16*)outs, (const uint32_t*)matrix, (const h16*)multiplier, (const h16*)scales,
                     (const h16*)zeros, B * M, K, S, g, false, st))
         return check_launch("matmul");
 

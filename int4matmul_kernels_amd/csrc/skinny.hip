@@ -1,4 +1,4 @@
-// Few-row product for gfx950: 2 .. 32 rows of states against a dense int4
+// Few-row product for gfx950: 2 .. 32 rows of states against a dense int4 / int3 / int2
 // weight matrix, HBM-bound like the matvec (every packed word is read once and
 // used for all rows).  The reference has no such path: it sends M >= 2 to its
 // 64-row matmul tiles (int4matmul.cpp:27) and M == 1 with B > 1 to one matvec
@@ -67,28 +67,63 @@ __device__ __forceinline__ uint32_t vgpr_const(uint32_t literal) {
     return r;
 }
 
-// k order of the 8 halves of an operand chunk
-__device__ constexpr int SK_ORDER[8] = {0, 4, 1, 5, 2, 6, 3, 7};
+// Per format: the k order of the 8 halves of an operand chunk, the offsets the
+// magic-number decode leaves on the low / high half of operand register e, and
+// the packed rows of a 32-row block.
+//   int4: order 0,4,1,5,2,6,3,7; registers 0, 2 carry 1024 + q, registers 1, 3 carry 64 + q
+//   int2: natural order, {1024 + q_even, 256 + q_odd};  int3: natural order, {1024 + q_even, 128 + q_odd}
+template <int BITS> struct SkFmt;
+template <> struct SkFmt<4> {
+    static constexpr int ROWS = 4, LOADS = 2;            // packed rows per block, loads per lane and unit
+    __device__ static constexpr int order(int e) { return (e >> 1) + 4 * (e & 1); }
+    __device__ static constexpr uint32_t offs(int e) { return (e & 1) ? 0x54005400u : 0x64006400u; }
+};
+template <> struct SkFmt<2> {
+    static constexpr int ROWS = 2, LOADS = 2;
+    __device__ static constexpr int order(int e) { return e; }
+    __device__ static constexpr uint32_t offs(int) { return 0x5C006400u; }
+};
+template <> struct SkFmt<3> {
+    static constexpr int ROWS = 3, LOADS = 4;
+    __device__ static constexpr int order(int e) { return e; }
+    __device__ static constexpr uint32_t offs(int) { return 0x58006400u; }
+};
 
-// packed word -> MFMA operand {1024 + q0, 1024 + q4, 64 + q1, 64 + q5, 1024 + q2, ...}
-__device__ __forceinline__ h16x8 magic_operand_int4(uint32_t u, uint32_t m0, uint32_t m1, uint32_t g0, uint32_t g1) {
-    const uint32_t u8 = u >> 8;
-    const u32x4 r = {(u & m0) | g0, (u & m1) | g1, (u8 & m0) | g0, (u8 & m1) | g1};
+// The 8 codes of one chunk (`f`: BITS bits apart, LSB first, garbage above) -> MFMA
+// operand of magic numbers; m0/g0 (and m1/g1 for int4) are the format's mask and
+// magic constants held in VGPRs.
+template <int BITS>
+__device__ __forceinline__ h16x8 magic_operand(uint32_t f, uint32_t m0, uint32_t m1, uint32_t g0, uint32_t g1) {
+    u32x4 r;
+    if constexpr (BITS == 4) {
+        const uint32_t f8 = f >> 8;
+        r = u32x4{(f & m0) | g0, (f & m1) | g1, (f8 & m0) | g0, (f8 & m1) | g1};
+    } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const uint32_t u = f >> (2 * BITS * e);
+            r[e] = (__builtin_amdgcn_perm(u, u, 0x01000100u) & m0) | g0;       // low 16 bits in both halves
+        }
+    }
     return bitcast<h16x8>(r);
 }
 
-__device__ __forceinline__ h16x8 exact_operand_int4(uint32_t u, h16 sc, h16 ze) {
+template <int BITS>
+__device__ __forceinline__ h16x8 exact_operand(uint32_t f, h16 sc, h16 ze) {
     h16x8 r;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) r[e] = dequant_code<4>((u >> (4 * SK_ORDER[e])) & 15u, sc, ze);
+    for (int e = 0; e < 8; ++e)
+        r[e] = dequant_code<BITS>((f >> (BITS * SkFmt<BITS>::order(e))) & ((1u << BITS) - 1u), sc, ze);
     return r;
 }
 
 // CW: columns per lane; RT: row groups of 8 that can hold real rows (R <= 8 RT);
 // MT: 16-row MFMA tiles; PF: units of packed weights in flight per wave
-template <int CW, int RT>
+template <int BITS, int CW, int RT>
 __global__ __launch_bounds__(512) void skinny_kernel(SkinnyArgs a) {
-    constexpr int PF = 4, MT = RT == 4 ? 2 : 1;
+    using F = SkFmt<BITS>;
+    constexpr int NL = F::LOADS;
+    constexpr int PF = BITS == 3 && CW == 4 ? 2 : 4, MT = RT == 4 ? 2 : 1;
     constexpr int PFX = RT == 4 ? 2 : 4;            // units of states in flight per wave
     constexpr int STRIP = 16 * CW;
     extern __shared__ __attribute__((aligned(16))) char lds[];
@@ -141,13 +176,28 @@ __global__ __launch_bounds__(512) void skinny_kernel(SkinnyArgs a) {
     if (u0 >= u1) general = scan_scales();          // idle waves still take part in its barriers
     if (u0 < u1) {
         // ---- loaders
-        // weights of unit u: packed rows 8u + 4 blk + h, blk = 0, 1, CW words each
-        const uint32_t* wbase = a.matrix + (int64_t)h * a.S + col0;
-        const int64_t wrow4 = (int64_t)4 * a.S;
-        auto load_w = [&](words_t w[2], int u) {
-            const uint32_t* p = wbase + (int64_t)u * 8 * a.S;
+        // weights of unit u, CW words per load.  Lane group h needs chunk h (8 codes) of
+        // each of the unit's two 32-row blocks:
+        //   int4: packed row 4 blk + h;  int2: row 2 blk + h / 2, its low or high half;
+        //   int3: bits 24 h .. 24 h + 23 of the block's 96-bit stream = rows {0,0,1,1}[h] and the
+        //         next one, shifted right by {0, 24, 16, 40}[h]
+        const int wrow = BITS == 4 ? h : (BITS == 2 ? (h >> 1) : (h >> 1));
+        const int wshift = BITS == 4 ? 0 : (BITS == 2 ? 16 * (h & 1) : (h == 0 ? 0 : h == 1 ? 24 : h == 2 ? 16 : 40));
+        const uint32_t* wbase = a.matrix + (int64_t)wrow * a.S + col0;
+        auto load_w = [&](words_t w[NL], int u) {
+            const uint32_t* p = wbase + (int64_t)u * (2 * F::ROWS) * a.S;
 #pragma unroll
-            for (int i = 0; i < 2; ++i) w[i] = __builtin_nontemporal_load(reinterpret_cast<const words_t*>(p + i * wrow4));
+            for (int i = 0; i < NL; ++i) {
+                const int row = BITS == 3 ? 3 * (i >> 1) + (i & 1) : F::ROWS * i;       // relative to the lane's first row
+                w[i] = __builtin_nontemporal_load(reinterpret_cast<const words_t*>(p + (int64_t)row * a.S));
+            }
+        };
+        // the 8 codes of chunk h of block blk, column c
+        auto chunk_bits = [&](const words_t w[NL], int blk, int c) -> uint32_t {
+            if constexpr (BITS == 3)
+                return (uint32_t)((((uint64_t)word_of<CW>(w[2 * blk + 1], c) << 32) | word_of<CW>(w[2 * blk], c)) >> wshift);
+            else
+                return word_of<CW>(w[blk], c) >> wshift;
         };
         // states of unit u (8 RT rows x 128 bytes): 8 / RT lanes per row, RT 16-byte chunks
         // each; the rows of the LDS buffers beyond 8 RT stay zero
@@ -162,18 +212,20 @@ __global__ __launch_bounds__(512) void skinny_kernel(SkinnyArgs a) {
         };
         // store a loaded unit to LDS buffer p and return its per-row sums (all lanes of a row get them)
         auto stage_x = [&](const u32x4 xr[RT], int p, float& sx, float& so) {
-            const uint32_t ONES = 0x3C003C00u, OFF_A = 0x64006400u, OFF_B = 0x54005400u;   // 1, 1024, 64
+            const uint32_t ONES = 0x3C003C00u;
             sx = 0.f; so = 0.f;
 #pragma unroll
             for (int i = 0; i < RT; ++i) {
                 const u32x4 v = xr[i];
-                // k order 0,4,1,5,2,6,3,7 inside the chunk, as the operand decode produces it
-                const u32x4 q = {__builtin_amdgcn_perm(v[2], v[0], 0x05040100u), __builtin_amdgcn_perm(v[2], v[0], 0x07060302u),
-                                 __builtin_amdgcn_perm(v[3], v[1], 0x05040100u), __builtin_amdgcn_perm(v[3], v[1], 0x07060302u)};
+                // the k order inside the chunk that the operand decode produces (int4: 0,4,1,5,2,6,3,7)
+                u32x4 q = v;
+                if constexpr (BITS == 4)
+                    q = u32x4{__builtin_amdgcn_perm(v[2], v[0], 0x05040100u), __builtin_amdgcn_perm(v[2], v[0], 0x07060302u),
+                              __builtin_amdgcn_perm(v[3], v[1], 0x05040100u), __builtin_amdgcn_perm(v[3], v[1], 0x07060302u)};
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     sx = dot2(q[e], ONES, sx);
-                    so = dot2(q[e], (e & 1) ? OFF_B : OFF_A, so);
+                    so = dot2(q[e], F::offs(e), so);
                 }
                 *reinterpret_cast<u32x4*>(my + p * SK_XBUF + xm * SK_PITCH + (xpart * RT + i) * 16) = q;
             }
@@ -186,10 +238,11 @@ __global__ __launch_bounds__(512) void skinny_kernel(SkinnyArgs a) {
         // rows that never receive states must read as zero
         for (int i = lane; i < 2 * SK_XBUF / 16; i += 64) *reinterpret_cast<u32x4*>(my + i * 16) = u32x4{0, 0, 0, 0};
 
-        words_t w[PF][2];
+        words_t w[PF][NL];
         u32x4 xr[PFX][RT];
-        const uint32_t m0 = vgpr_const(0x000F000Fu), m1 = vgpr_const(0x00F000F0u);
-        const uint32_t g0 = vgpr_const(0x64006400u), g1 = vgpr_const(0x54005400u);
+        const uint32_t m0 = vgpr_const(BITS == 4 ? 0x000F000Fu : BITS == 2 ? 0x000C0003u : 0x00380007u);
+        const uint32_t g0 = vgpr_const(BITS == 4 ? 0x64006400u : BITS == 2 ? 0x5C006400u : 0x58006400u);
+        const uint32_t m1 = BITS == 4 ? vgpr_const(0x00F000F0u) : 0u, g1 = BITS == 4 ? vgpr_const(0x54005400u) : 0u;
         float gS = 0.f, gO = 0.f;           // sums of the current group so far (row lane / 2)
         float nS, nO;                       // sums of the unit staged last (the next to be multiplied)
         // scale / zero of the lane's CW columns for group gi, from the LDS copy
@@ -222,7 +275,7 @@ __global__ __launch_bounds__(512) void skinny_kernel(SkinnyArgs a) {
 
         // p: parity of the LDS buffer that holds unit u; xn: the register set with the states of unit u + 1.
         // The decode mode is a compile-time tag: one loop body per mode, no branches inside.
-        auto step = [&](auto mode, int u, int p, words_t w[2], u32x4 xn[RT]) {
+        auto step = [&](auto mode, int u, int p, words_t w[NL], u32x4 xn[RT]) {
             constexpr bool general = decltype(mode)::value;
             if constexpr (general) {
                 if (u == u0 || u % a.group_units == 0) load_sz(u / a.group_units);
@@ -237,9 +290,9 @@ __global__ __launch_bounds__(512) void skinny_kernel(SkinnyArgs a) {
                     xa[mt] = *reinterpret_cast<const h16x8*>(my + p * SK_XBUF + (j + 16 * mt) * SK_PITCH + (i * 4 + h) * 16);
 #pragma unroll
                 for (int c = 0; c < CW; ++c) {
-                    const uint32_t word = word_of<CW>(w[i], c);
-                    const h16x8 wb = general ? exact_operand_int4(word, sc[c], ze[c])
-                                             : magic_operand_int4(word, m0, m1, g0, g1);
+                    const uint32_t f = chunk_bits(w, i, c);
+                    const h16x8 wb = general ? exact_operand<BITS>(f, sc[c], ze[c])
+                                             : magic_operand<BITS>(f, m0, m1, g0, g1);
 #pragma unroll
                     for (int mt = 0; mt < MT; ++mt)
                         acc[c][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[mt], wb, acc[c][mt], 0, 0, 0);
@@ -273,11 +326,12 @@ __global__ __launch_bounds__(512) void skinny_kernel(SkinnyArgs a) {
             }
         };
         auto run = [&](auto mode) {
-            for (int u = u0; u < u1; u += PF) {
+            constexpr int UN = PF > PFX ? PF : PFX;      // register sets rotate with periods PF and PFX
+            for (int u = u0; u < u1; u += UN) {
 #pragma unroll
-                for (int f = 0; f < PF; ++f) {
+                for (int f = 0; f < UN; ++f) {
                     if (f > 0 && u + f >= u1) break;
-                    step(mode, u + f, f & 1, w[f], xr[(f + 1) % PFX]);
+                    step(mode, u + f, f & 1, w[f % PF], xr[(f + 1) % PFX]);
                 }
             }
         };
@@ -331,7 +385,7 @@ __global__ __launch_bounds__(512) void skinny_kernel(SkinnyArgs a) {
     }
 }
 
-template <int CW>
+template <int BITS, int CW>
 static bool launch_skinny(const SkinnyArgs& a, int waves, hipStream_t st) {
     const int strips = a.S / (16 * CW);
     const int rt = (a.R + 7) / 8;
@@ -354,15 +408,22 @@ static bool launch_skinny(const SkinnyArgs& a, int waves, hipStream_t st) {
         }
         hipLaunchKernelGGL(kernel, grid, block, lds, st, a);
     };
-    if (rt <= 1) go(skinny_kernel<CW, 1>, 0);
-    else if (rt <= 2) go(skinny_kernel<CW, 2>, 1);
-    else go(skinny_kernel<CW, 4>, 2);
+    if (rt <= 1) go(skinny_kernel<BITS, CW, 1>, 0);
+    else if (rt <= 2) go(skinny_kernel<BITS, CW, 2>, 1);
+    else go(skinny_kernel<BITS, CW, 4>, 2);
     return true;
 }
 
-// Product of R <= 32 rows with a dense int4 matrix.  Returns false when the shape
-// is not one this kernel takes (the caller then uses the general kernels).
-bool skinny_int4(h16* outs, const uint32_t* matrix, const h16* x, const h16* scales, const h16* zeros,
+template <int BITS>
+static bool launch_skinny_cw(const SkinnyArgs& a, int cw, int waves, hipStream_t st) {
+    if (cw == 4) return launch_skinny<BITS, 4>(a, waves, st);
+    if (cw == 2) return launch_skinny<BITS, 2>(a, waves, st);
+    return launch_skinny<BITS, 1>(a, waves, st);
+}
+
+// Product of R <= 32 rows with a dense matrix.  Returns false when the shape is
+// not one this kernel takes (the caller then uses the general kernels).
+bool skinny_dense(int bits, h16* outs, const uint32_t* matrix, const h16* x, const h16* scales, const h16* zeros,
                  int64_t R, int64_t K, int64_t S, int64_t group_size, bool accumulate, hipStream_t st) {
     if (R < 2 || R > 32 || S % 16 != 0 || K % 64 != 0 || K > (1 << 30) || S > (1 << 28)) return false;
     SkinnyArgs a;
@@ -384,9 +445,9 @@ bool skinny_int4(h16* outs, const uint32_t* matrix, const h16* x, const h16* sca
     if (waves != 2 && waves != 4 && waves != 8) waves = S / (16 * cw) >= 256 ? 4 : 8;
     while (waves > 1 && units < 2 * waves) waves >>= 1;
     a.units_per_wave = (units + waves - 1) / waves;
-    if (cw == 4) return launch_skinny<4>(a, waves, st);
-    if (cw == 2) return launch_skinny<2>(a, waves, st);
-    return launch_skinny<1>(a, waves, st);
+    if (bits == 4) return launch_skinny_cw<4>(a, cw, waves, st);
+    if (bits == 3) return launch_skinny_cw<3>(a, cw, waves, st);
+    return launch_skinny_cw<2>(a, cw, waves, st);
 }
 
 }  // namespace i4

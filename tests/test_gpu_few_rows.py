@@ -1,4 +1,4 @@
-"""The few-row kernel (2 .. 32 rows of states in all, dense int4): every packed
+"""The few-row kernel (2 .. 32 rows of states in all, dense formats): every packed
 word is read once for all rows.  It serves `quant_matmul` with small M (any
 batch layout that flattens to <= 32 rows) and the matvec entry with B > 1.
 Its numerics are the matvec's (exact sum of x (q - z) s, no per-weight fp16
@@ -27,10 +27,18 @@ def _check(H, p, kind, prior=None):
     return d, got
 
 
+def _problem(bits, **kw):
+    if bits != 4:       # scales U(0.004, 0.08), zero at the mid-code
+        kw.setdefault("scale_range", (0.004, 0.08))
+        kw.setdefault("zero_const", 3.5 if bits == 3 else 1.5)
+    return O.make_problem(bits=bits, **kw)
+
+
+@pytest.mark.parametrize("bits", [4, 3, 2])
 @pytest.mark.parametrize("M", [2, 3, 8, 9, 16, 17, 31, 32])
-@pytest.mark.parametrize("K,S,g", [(512, 256, 128), (64, 64, 64), (1024, 192, -1), (320, 1024, 64)])
-def test_few_rows_matmul(H, M, K, S, g):
-    p = O.make_problem(K=K, S=S, M=M, bits=4, group_size=g, seed=M + K)
+@pytest.mark.parametrize("K,S,g", [(512, 256, 128), (64, 64, 64), (1024, 192, -1), (320, 1024, 64), (256, 8192, 128)])
+def test_few_rows_matmul(H, bits, M, K, S, g):
+    p = _problem(bits, K=K, S=S, M=M, group_size=g, seed=M + K)
     junk = np.full((1, M, S), -77.0, np.float16)
     d, got = _check(H, p, "mtx", prior=junk)                      # matmul semantics: prior contents overwritten
     # against the general kernel it replaces
@@ -42,9 +50,10 @@ def test_few_rows_matmul(H, M, K, S, g):
     assert O.max_rel_error(ref.astype(np.float64), got) < H.TOL_EXACT
 
 
+@pytest.mark.parametrize("bits", [4, 3, 2])
 @pytest.mark.parametrize("B,M", [(2, 1), (5, 1), (32, 1), (4, 4), (3, 7)])
-def test_few_rows_batches_flatten(H, B, M):
-    p = O.make_problem(K=768, S=320, M=M, bits=4, group_size=128, seed=B * 10 + M, B=B)
+def test_few_rows_batches_flatten(H, bits, B, M):
+    p = _problem(bits, K=768, S=320, M=M, group_size=128, seed=B * 10 + M, B=B)
     _check(H, p, "mtx")
     if M == 1:
         # the matvec entry adds onto the prior contents of outs
@@ -52,24 +61,27 @@ def test_few_rows_batches_flatten(H, B, M):
         _check(H, p, "vec", prior=prior)
 
 
-def test_few_rows_exponent_mode_columns(H):
-    p = O.make_problem(K=512, S=256, M=6, bits=4, group_size=128, seed=9)
+@pytest.mark.parametrize("bits", [4, 3, 2])
+def test_few_rows_exponent_mode_columns(H, bits):
+    p = _problem(bits, K=512, S=256, M=6, group_size=128, seed=9)
     p["scales"][1, 40:48] *= np.float16(-1)                   # one strip switches to the exact decode
     p["scales"][3, 200] *= np.float16(-1)
     _check(H, p, "mtx")
 
 
-def test_few_rows_degenerate_known_answer(H):
+@pytest.mark.parametrize("bits", [4, 3, 2])
+def test_few_rows_degenerate_known_answer(H, bits):
     K, S, M = 1024, 128, 12
     codes = np.ones((K, S), np.uint8)
-    p = dict(B=1, M=M, S=S, K=K, bits=4, group_size=128, matrix=O.pack_dense(4, codes), sparse_mask=None,
+    p = dict(B=1, M=M, S=S, K=K, bits=bits, group_size=128, matrix=O.pack_dense(bits, codes), sparse_mask=None,
              states=np.ones((1, M, K), np.float16), scales=np.ones((K // 128, S), np.float16),
              zeros=np.zeros((K // 128, S), np.float16))
     got = H.run_capi(p, H.dev_problem(p), "mtx")
     assert np.all(got.astype(np.float64) == K)
 
 
-def test_few_rows_full_size(H):
+@pytest.mark.parametrize("bits", [4, 3, 2])
+def test_few_rows_full_size(H, bits):
     """K=5120, S=20480, 16 rows: the whole output against the oracle"""
-    p = O.make_problem(K=5120, S=20480, M=16, bits=4, group_size=128, seed=4)
+    p = _problem(bits, K=5120, S=20480, M=16, group_size=128, seed=4)
     _check(H, p, "mtx")
