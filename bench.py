@@ -64,7 +64,7 @@ def main():
     K, S, g, NSETS = 5120, 20480, 128, 7
     steps, warmup = max(1, args.steps), max(0, args.warmup)
 
-    # ---- seeded synthetic workload (BASELINE config 2); set 0 is the oracle's problem
+    # ---- seeded synthetic workload (the headline matvec shape); set 0 is the oracle's problem
     p = O.make_problem(K=K, S=S, M=1, bits=4, group_size=g, seed=0)
     gen = torch.Generator(device="cpu").manual_seed(0)
     sets = []
@@ -143,7 +143,7 @@ def main():
         torch.cuda.synchronize()
         result["calibration"] = {"kernel": "torch device copy", "bytes_read": 256 << 20, "bytes_written": 256 << 20}
 
-    # ---- the matmul half of the metric: M=2048, same weights (BASELINE config 3)
+    # ---- the matmul half of the metric: M=2048, same weights (the headline matmul shape)
     if not args.no_gemm:
         M = 2048
         xs = torch.randn((1, M, K), generator=torch.Generator(device="cpu").manual_seed(1)).half().to(dev)

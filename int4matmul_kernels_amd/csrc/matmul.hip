@@ -3,18 +3,20 @@
 // where w16 is the fp16 matrix the reference's unpack step builds (two fp16
 // roundings per weight in linear mode, one fused multiply-add in exponent mode).
 //
-// One workgroup owns a BM x BN tile of outs and walks K in steps of 64.  Per
-// step the packed weights of the tile (64 x BN codes) are read from HBM once,
-// decoded and dequantised to fp16 ONCE by the workgroup and stored to LDS in
-// the operand layout of v_mfma_f32_32x32x16_f16: 16-byte chunks of 8
-// consecutive k for one column, chunk (kc, n) at kc*BN + n, which both the
+// Two kernels.  matmul_kernel_pipe (further down) is the fast one for shapes
+// made of whole tiles; matmul_kernel takes everything else.  Common to both: one
+// workgroup owns a tile of outs; per K step the packed weights of the tile are
+// read from HBM once, decoded and dequantised to fp16 ONCE by the workgroup and
+// stored to LDS in the operand layout of v_mfma_f32_32x32x16_f16: 16-byte chunks
+// of 8 consecutive k for one column, chunk (kc, n) at kc*BN + n, which both the
 // writes (lanes along n) and the MFMA operand reads (lanes along n) touch
-// without bank conflicts.  The states tile (BM x 64 fp16) is stored row-major
-// with an XOR swizzle of the chunk index so that row-contiguous writes and
-// column-of-rows operand reads are both conflict-free.  Accumulation is fp32 in
-// the MFMA accumulators.  Global loads of step k+1 are issued before the MFMA
-// phase of step k (register prefetch); two workgroups share a CU so that one
-// decodes while the other multiplies.
+// without bank conflicts.  The states tile is stored row-major with an XOR
+// swizzle of the chunk index so that row-contiguous writes and column-of-rows
+// operand reads are both conflict-free.  Accumulation is fp32 in the MFMA
+// accumulators.
+//
+// matmul_kernel walks K in steps of 64 with the global loads of step k+1 issued
+// before the MFMA phase of step k (register prefetch) and two barriers per step.
 //
 // Workgroups are renumbered so that the 8 XCDs (each with its own L2) take
 // disjoint column ranges of the weight matrix.
@@ -720,6 +722,7 @@ static void launch(const MatmulArgs& a, int64_t B, hipStream_t st) {
     const bool m_ok = (m_pad - a.M) * 8 <= a.M && a.K <= (1 << 22) && a.S <= (1 << 27);
     const bool pipe2_ok = !SPARSE && m_ok && a.S % 128 == 0;
     const bool pipe4_ok = m_ok && a.S % 256 == 0;
+    if (variant != 1 && variant != 3 && variant != 5 && variant != 6) variant = 0;
     if ((variant == 5 && !pipe2_ok) || (variant == 6 && !pipe4_ok)) variant = 0;
     if (variant == 0) {
         const int64_t tiles4 = m_pad / 256 * (a.S / 256) * B;
@@ -731,9 +734,7 @@ static void launch(const MatmulArgs& a, int64_t B, hipStream_t st) {
         else variant = 1;
     }
     if (variant == 1) launch_tile<BITS, SPARSE, 128, 128, 64, 64>(a, B, st);
-    else if (variant == 2) launch_tile<BITS, SPARSE, 128, 256, 64, 128>(a, B, st);
     else if (variant == 3) launch_tile<BITS, SPARSE, 128, 256, 128, 64>(a, B, st);
-    else if (variant == 4) launch_tile<BITS, SPARSE, 256, 256, 128, 64>(a, B, st);
     else if (variant == 6) launch_pipe<BITS, SPARSE, 4>(a, B, st);
     else if constexpr (!SPARSE) launch_pipe<BITS, false, 2>(a, B, st);
 }

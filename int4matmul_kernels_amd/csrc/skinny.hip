@@ -8,10 +8,12 @@
 // rows of states as its 16 x 32 operand (rows >= R are zero; 17 .. 32 rows take
 // two such tiles) and, as its 32 x 16 operand, 8 consecutive k of one column per
 // lane -- which is exactly one packed int4 word; the four lane groups of a wave
-// hold the four packed rows of a 32-row block.  A word becomes that operand without converting a single code:
-// mask-and-OR of the word (and of the word shifted by 8) gives the half2 pairs
-// {1024 + q0, 1024 + q4}, {64 + q1, 64 + q5}, {1024 + q2, 1024 + q6}, {64 + q3,
-// 64 + q7}; the states are stored to LDS in the same k order 0,4,1,5,2,6,3,7.
+// hold the four packed rows of a 32-row block.  A word becomes that operand
+// without converting a single code: mask-and-OR of the word (and of the word
+// shifted by 8) gives the half2 pairs {1024 + q0, 1024 + q4}, {64 + q1, 64 + q5},
+// {1024 + q2, 1024 + q6}, {64 + q3, 64 + q7}; the states are stored to LDS in the
+// same k order 0,4,1,5,2,6,3,7.  (int2 / int3: the chunk's 16 / 24 bits, pairs
+// {1024 + q_even, 256 or 128 + q_odd} in natural order.)
 // The offsets are removed once per quantisation group in fp32 together with
 // scale and zero:
 //     y[m, n] += s[n] * (acc[m, n] - sum_k off_k x[m, k] - z[n] * sum_k x[m, k])

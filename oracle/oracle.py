@@ -302,7 +302,7 @@ def max_rel_error(truth: np.ndarray, cand: np.ndarray, floor_frac: float = 1.0) 
 
 
 # --------------------------------------------------------------------------
-# Seeded synthetic workloads (BASELINE configs).  Generated with numpy on the
+# Seeded synthetic workloads of the benchmark shapes.  Generated with numpy on the
 # CPU so that every machine sees identical bits.
 # --------------------------------------------------------------------------
 def make_problem(K, S, M=1, bits=4, group_size=128, sparse=False, seed=0, B=1,

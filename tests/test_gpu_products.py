@@ -19,7 +19,7 @@ def H():
 
 
 def _problem(bits, sparse, **kw):
-    if bits != 4:       # BASELINE config 5: scales U(0.004, 0.08), zero at the mid-code
+    if bits != 4:       # int3 / int2 benchmark configuration: scales U(0.004, 0.08), zero at the mid-code
         kw.setdefault("scale_range", (0.004, 0.08))
         kw.setdefault("zero_const", 3.5 if bits == 3 else 1.5)
     return O.make_problem(bits=bits, sparse=sparse, **kw)
@@ -157,9 +157,9 @@ def test_single_group_accepts_1d_scales(H):
             H.assert_product_close(got[:, m:m + 1], exact, f32, kind="vec" if M == 1 else "mtx")
 
 
-# ------------------------------------------------- full-size BASELINE shapes
+# ------------------------------------------------- full-size benchmark shapes
 def test_full_size_matvec_and_matmul_c2_c3(H):
-    """K=5120, S=20480, g=128 (BASELINE configs 2 and 3): the matvec against the
+    """K=5120, S=20480, g=128 (the headline matvec and matmul shapes): the matvec against the
     oracle on every output; the M=2048 matmul on 24 sampled rows against the
     oracle, plus row-linearity of the whole product (a size-independent
     property: the product of a sum of two row blocks equals the sum of products
