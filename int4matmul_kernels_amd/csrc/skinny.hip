@@ -1,4 +1,4 @@
-// Few-row product for gfx950: 2 .. 32 rows of states against a dense int4 / int3 / int2
+// Few-row product for gfx950: 2 .. 96 rows of states (32 per workgroup) against a dense int4 / int3 / int2
 // weight matrix, HBM-bound like the matvec (every packed word is read once and
 // used for all rows).  The reference has no such path: it sends M >= 2 to its
 // 64-row matmul tiles (int4matmul.cpp:27) and M == 1 with B > 1 to one matvec
@@ -136,6 +136,9 @@ __global__ __launch_bounds__(512) void skinny_kernel(SkinnyArgs a) {
     const int col0 = blockIdx.x * STRIP + CW * j;              // first of this lane's CW columns
     const int units = a.K / 64;
     const int u0 = wave * a.units_per_wave, u1 = min(units, u0 + a.units_per_wave);
+    // more than 32 rows: blockIdx.y takes rows 32 y .. 32 y + 31 (each block reads the strip's weights again)
+    const int row0 = blockIdx.y * 32;
+    const int R = min(32, a.R - row0);
 
     // The strip's scales and zeros ([groups][STRIP] halves each) are copied to LDS
     // once: the loop then never waits on a global load other than its prefetched
@@ -205,8 +208,8 @@ __global__ __launch_bounds__(512) void skinny_kernel(SkinnyArgs a) {
         // each; the rows of the LDS buffers beyond 8 RT stay zero
         constexpr int LPR = 8 / RT;                                   // lanes per row
         const int xm = lane / LPR, xpart = lane % LPR;
-        const bool xreal = xm < a.R;
-        const h16* xsrc = a.x + (int64_t)min(xm, a.R - 1) * a.K + xpart * (8 * RT);
+        const bool xreal = xm < R;
+        const h16* xsrc = a.x + (int64_t)(row0 + min(xm, R - 1)) * a.K + xpart * (8 * RT);
         auto load_x = [&](u32x4 xr[RT], int u) {
 #pragma unroll
             for (int i = 0; i < RT; ++i)
@@ -374,8 +377,8 @@ __global__ __launch_bounds__(512) void skinny_kernel(SkinnyArgs a) {
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 const int m = mt * 16 + 4 * h + e;
-                if (m < a.R) {
-                    h16* o = a.outs + (int64_t)m * a.S + col0;
+                if (m < R) {
+                    h16* o = a.outs + (int64_t)(row0 + m) * a.S + col0;
 #pragma unroll
                     for (int c = 0; c < CW; ++c) {
                         float v = y[c][mt][e];
@@ -390,13 +393,13 @@ __global__ __launch_bounds__(512) void skinny_kernel(SkinnyArgs a) {
 template <int BITS, int CW>
 static bool launch_skinny(const SkinnyArgs& a, int waves, hipStream_t st) {
     const int strips = a.S / (16 * CW);
-    const int rt = (a.R + 7) / 8;
+    const int rt = ((a.R > 32 ? 32 : a.R) + 7) / 8;
     const int groups = (a.K / 64 + a.group_units - 1) / a.group_units;
     size_t lds = (size_t)waves * SK_WAVE_LDS + 16 + (size_t)groups * 16 * CW * 4;
     const size_t red = (size_t)(waves / 2) * (rt <= 2 ? 1 : 2) * 16 * 16 * CW * 4;
     if (red > lds) lds = red;
     if (lds > 150 * 1024) return false;
-    const dim3 grid(strips), block(waves * 64);
+    const dim3 grid(strips, (a.R + 31) / 32), block(waves * 64);
     auto go = [&](auto kernel, int slot) {
         // more than 64 KB of dynamic LDS has to be requested once per kernel and device
         static std::atomic<uint64_t> done[3];
@@ -423,11 +426,11 @@ static bool launch_skinny_cw(const SkinnyArgs& a, int cw, int waves, hipStream_t
     return launch_skinny<BITS, 1>(a, waves, st);
 }
 
-// Product of R <= 32 rows with a dense matrix.  Returns false when the shape is
+// Product of R <= 96 rows with a dense matrix (beyond that the tile kernels are faster).  Returns false when the shape is
 // not one this kernel takes (the caller then uses the general kernels).
 bool skinny_dense(int bits, h16* outs, const uint32_t* matrix, const h16* x, const h16* scales, const h16* zeros,
                  int64_t R, int64_t K, int64_t S, int64_t group_size, bool accumulate, hipStream_t st) {
-    if (R < 2 || R > 32 || S % 16 != 0 || K % 64 != 0 || K > (1 << 30) || S > (1 << 28)) return false;
+    if (R < 2 || R > 96 || S % 16 != 0 || K % 64 != 0 || K > (1 << 30) || S > (1 << 28)) return false;
     SkinnyArgs a;
     a.outs = outs; a.matrix = matrix; a.x = x; a.scales = scales; a.zeros = zeros;
     a.R = (int)R; a.K = (int)K; a.S = (int)S;

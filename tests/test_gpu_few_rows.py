@@ -1,4 +1,4 @@
-"""The few-row kernel (2 .. 32 rows of states in all, dense formats): every packed
+"""The few-row kernel (2 .. 96 rows of states in all, dense formats): every packed
 word is read once for all rows.  It serves `quant_matmul` with small M (any
 batch layout that flattens to <= 32 rows) and the matvec entry with B > 1.
 Its numerics are the matvec's (exact sum of x (q - z) s, no per-weight fp16
@@ -35,7 +35,7 @@ def _problem(bits, **kw):
 
 
 @pytest.mark.parametrize("bits", [4, 3, 2])
-@pytest.mark.parametrize("M", [2, 3, 8, 9, 16, 17, 31, 32])
+@pytest.mark.parametrize("M", [2, 3, 8, 9, 16, 17, 31, 32, 33, 64, 71, 96])
 @pytest.mark.parametrize("K,S,g", [(512, 256, 128), (64, 64, 64), (1024, 192, -1), (320, 1024, 64), (256, 8192, 128)])
 def test_few_rows_matmul(H, bits, M, K, S, g):
     p = _problem(bits, K=K, S=S, M=M, group_size=g, seed=M + K)
@@ -51,7 +51,7 @@ def test_few_rows_matmul(H, bits, M, K, S, g):
 
 
 @pytest.mark.parametrize("bits", [4, 3, 2])
-@pytest.mark.parametrize("B,M", [(2, 1), (5, 1), (32, 1), (4, 4), (3, 7)])
+@pytest.mark.parametrize("B,M", [(2, 1), (5, 1), (32, 1), (4, 4), (3, 7), (40, 1), (5, 17), (96, 1)])
 def test_few_rows_batches_flatten(H, bits, B, M):
     p = _problem(bits, K=768, S=320, M=M, group_size=128, seed=B * 10 + M, B=B)
     _check(H, p, "mtx")
