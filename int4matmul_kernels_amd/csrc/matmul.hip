@@ -716,10 +716,11 @@ static void launch(const MatmulArgs& a, int64_t B, hipStream_t st) {
     // needs more registers than the four-wave shape leaves).  Everything else:
     // 128 x 256 tiles, and 128 x 128 for narrow outputs or few rows.
     int variant = (int)tuning(TUNE_MM_VARIANT);
-    // (M is padded to whole tiles; worth it while the padding stays below an eighth of M)
+    // (M is padded to whole tiles; worth it while the padding stays below an eighth of M,
+    // and for a single row of tiles from 161 rows on)
     const int64_t m_pad = (a.M + 255) / 256 * 256;
     // (the kernel's per-lane byte offsets are 32-bit: 256 rows of states, 4 packed rows of weights)
-    const bool m_ok = (m_pad - a.M) * 8 <= a.M && a.K <= (1 << 22) && a.S <= (1 << 27);
+    const bool m_ok = ((m_pad - a.M) * 8 <= a.M || (a.M > 160 && a.M <= 256)) && a.K <= (1 << 22) && a.S <= (1 << 27);
     const bool pipe2_ok = !SPARSE && m_ok && a.S % 128 == 0;
     const bool pipe4_ok = m_ok && a.S % 256 == 0;
     if (variant != 1 && variant != 3 && variant != 5 && variant != 6) variant = 0;
