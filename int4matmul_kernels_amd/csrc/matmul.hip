@@ -41,6 +41,7 @@ struct MatmulArgs {
     int M, K, S;
     int group_units;        // group size / 64
     int tiles_m, tiles_n;
+    int by_columns;         // pipelined kernel: 1 = an XCD walks its range of tile columns row by row
 };
 
 // Raw packed data of one (32-row block, column) cell
@@ -691,8 +692,26 @@ __global__ __launch_bounds__(NW * 128, NW == 2 ? 2 : 1) void matmul_kernel_pipe(
     __shared__ __attribute__((aligned(16))) uint32_t Lut[SPARSE ? SPARSE_LUT_WORDS : 4];
     int bid = blockIdx.x;
     const int total = a.tiles_m * a.tiles_n;
-    if (total % 8 == 0) bid = (bid % 8) * (total / 8) + bid / 8;     // XCD-aware renumbering
-    const int tile_m = bid % a.tiles_m, tile_n = bid / a.tiles_m;
+    int tile_m, tile_n;
+    if (total % 8 == 0) {
+        // XCD-aware numbering: workgroups are dealt round-robin to the 8 XCDs (each
+        // with its own L2), so XCD x takes the contiguous range x * total / 8 ... of tiles
+        const int per_xcd = total / 8, l = bid / 8;
+        if (a.by_columns) {
+            // ... walked one tile row at a time across the XCD's tile columns: the tiles in
+            // flight on an XCD then share few rows of states, whose 64 bytes per row and K
+            // step outweigh the packed weights' 16 bytes per column (measured: 1-5 % faster
+            // than column by column)
+            const int cols = per_xcd / a.tiles_m;
+            tile_m = l / cols;
+            tile_n = (bid % 8) * cols + l % cols;
+        } else {
+            bid = (bid % 8) * per_xcd + l;
+            tile_m = bid % a.tiles_m, tile_n = bid / a.tiles_m;
+        }
+    } else {
+        tile_m = bid % a.tiles_m, tile_n = bid / a.tiles_m;
+    }
     const int64_t boff = blockIdx.z;
     pipe_tile<BITS, SPARSE, TM, NW>(a, tile_m * BM, tile_n * BN, a.x + boff * a.M * (int64_t)a.K,
                                    a.outs + boff * a.M * (int64_t)a.S, As, Bs, Lut);
@@ -703,6 +722,7 @@ static void launch_pipe(MatmulArgs a, int64_t B, hipStream_t st) {
     a.tiles_m = (a.M + TM * 64 - 1) / (TM * 64);
     a.tiles_n = a.S / (NW * 64);
     const dim3 grid(a.tiles_m * a.tiles_n, 1, (unsigned)B), block(NW * 128);
+    a.by_columns = a.tiles_n % 8 == 0;
     hipLaunchKernelGGL((matmul_kernel_pipe<BITS, SPARSE, NW, TM>), grid, block, 0, st, a);
 }
 
@@ -784,6 +804,7 @@ extern "C" int int4mm_matmul(int bits, void* outs, const void* matrix, const voi
     a.S = (int)S;
     a.group_units = (int)(g / 64 > 0x7FFFFFF ? 0x7FFFFFF : g / 64);
     a.tiles_m = a.tiles_n = 0;
+    a.by_columns = 0;
 
     if (sparse_mask) launch<4, true>(a, B, st);
     else if (bits == 4) launch<4, false>(a, B, st);
