@@ -58,7 +58,7 @@ template <int BITS, bool SPARSE> struct Fmt;
 template <> struct Fmt<4, false> { static constexpr int ROWS = 8, MROWS = 0, XS = 128; static constexpr bool FAST = true; };
 template <> struct Fmt<3, false> { static constexpr int ROWS = 6, MROWS = 0, XS = 160; static constexpr bool FAST = true; };
 template <> struct Fmt<2, false> { static constexpr int ROWS = 4, MROWS = 0, XS = 128; static constexpr bool FAST = true; };
-template <> struct Fmt<4, true>  { static constexpr int ROWS = 4, MROWS = 2, XS = 256; static constexpr bool FAST = true; };
+template <> struct Fmt<4, true>  { static constexpr int ROWS = 4, MROWS = 2, XS = 128; static constexpr bool FAST = true; };
 
 template <int BITS, bool SPARSE>
 struct Unit {
@@ -230,22 +230,27 @@ __host__ __device__ constexpr uint32_t pair_selector(int a, int b) {
 // 16:32 sparse int4.  Per (32-row block, column): a mask word and 16 kept codes
 // packed in 64 bits.  Two dot products are needed per column: A = sum over kept
 // rows of x*q and M = sum over kept rows of x (dropped rows contribute exactly 0).
-//  * M treats the mask word as 32 one-bit codes: (m >> 4i) & (0x00010001 << o) |
-//    magic gives the half2 {2^(10-o) + bit(4i+o), 2^(10-o) + bit(16+4i+o)}.
-//  * A first expands the kept codes to their rows.  The mask is taken a byte at
-//    a time: the next eight nibbles of the code stream are split into eight
-//    bytes (even / odd nibbles of one word), and a 256-entry table in LDS holds,
-//    for every mask byte, the four v_perm selectors that route the right code
-//    byte (or zero) into the 16-bit halves of the pairs (row j, row j+4) of that
-//    byte's eight rows; OR-ing 0x6400 into both halves makes them 1024 + q.
-// Staged states per unit: for each block 16 dwords {x_j, x_j+4} ordered as the
-// dense int4 path, then for each block 16 dwords {x_p, x_p+16}.
-__device__ __forceinline__ void unit_fast_sparse(const Unit<4, true>& u, const h16* xp, const u32x4* lut,
+// The kept codes are first expanded to their rows.  The mask is taken a byte at
+// a time: the next eight nibbles of the code stream are split into eight bytes
+// (even / odd nibbles of one word, each with bit 4 set as a "kept" flag), and a
+// 256-entry table in LDS holds, for every mask byte, the four v_perm selectors
+// that route the right byte (or zero) into the 16-bit halves of the pairs
+// (row j, row j+4) of that byte's eight rows.  The halves {0x001q, 0x001q'} go to
+// the MFMA as they are: as fp16 they are the denormals (16 + q) * 2^-24, which
+// the matrix unit multiplies exactly (it does not flush them).  Masking the same
+// halves with 0x0010 gives 16 * 2^-24 per kept row for the second dot product:
+//     accA = 2^-24 (A + 16 M),   accM = 2^-20 M.
+// The mask byte is first replicated into all four bytes of a register: its
+// population count is then the stream's shift in bits (4 per kept code), and its
+// bits 4..11 are the table offset (entries are stored under the nibble-swapped byte).
+// Staged states per unit: for each block 16 dwords {x_j, x_j+4}, ordered as the
+// dense int4 path.
+constexpr int SPARSE_LUT_BYTES = 256 * 16;
+
+__device__ __forceinline__ void unit_fast_sparse(const Unit<4, true>& u, const h16* xp, const char* lut,
                                                  f32x4 accA[4], f32x4 accM[4]) {
-    const uint32_t NIB = in_vgpr(0x0F0F0F0Fu), G10 = in_vgpr(0x64006400u);
-    const uint32_t B0 = in_vgpr(0x00010001u), B1 = in_vgpr(0x00020002u), B2 = in_vgpr(0x00040004u),
-                   B3 = in_vgpr(0x00080008u);
-    const uint32_t G9 = in_vgpr(0x60006000u), G8 = in_vgpr(0x5C005C00u), G7 = in_vgpr(0x58005800u);
+    const uint32_t NIB = in_vgpr(0x0F0F0F0Fu), FLAG = in_vgpr(0x10101010u), KEPT = in_vgpr(0x00100010u);
+    const uint32_t IDX = in_vgpr(0x00000FF0u);
     const uint32_t* xw = reinterpret_cast<const uint32_t*>(xp);
 #pragma unroll
     for (int hb = 0; hb < 2; ++hb) {
@@ -256,24 +261,21 @@ __device__ __forceinline__ void unit_fast_sparse(const Unit<4, true>& u, const h
             f32x4 ra = accA[c], rm = accM[c];
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                // ---- rows 8i .. 8i+7: expand and accumulate x*q
-                const uint32_t mb = (m >> (8 * i)) & 0xFFu;
-                const u32x4 sel = lut[mb];
+                // ---- rows 8i .. 8i+7
+                const uint32_t mb4 = __builtin_amdgcn_perm(m, m, 0x01010101u * i);      // mask byte i, four times
+                const u32x4 sel = *reinterpret_cast<const u32x4*>(lut + (mb4 & IDX));
                 const uint32_t chunk = (uint32_t)stream;
-                const uint32_t even = chunk & NIB, odd = (chunk >> 4) & NIB;
-                stream >>= 4 * __builtin_popcount(mb);
+                const uint32_t even = and_or(chunk, NIB, FLAG), odd = and_or(chunk >> 4, NIB, FLAG);
+                stream >>= __builtin_popcount(mb4);
                 const u32x4 px = *reinterpret_cast<const u32x4*>(xw + hb * 16 + i * 4);
-                const uint32_t b0 = __builtin_amdgcn_perm(odd, even, sel.x) | G10;
-                const uint32_t b1 = __builtin_amdgcn_perm(odd, even, sel.y) | G10;
-                const uint32_t b2 = __builtin_amdgcn_perm(odd, even, sel.z) | G10;
-                const uint32_t b3 = __builtin_amdgcn_perm(odd, even, sel.w) | G10;
+                const uint32_t b0 = __builtin_amdgcn_perm(odd, even, sel.x);
+                const uint32_t b1 = __builtin_amdgcn_perm(odd, even, sel.y);
+                const uint32_t b2 = __builtin_amdgcn_perm(odd, even, sel.z);
+                const uint32_t b3 = __builtin_amdgcn_perm(odd, even, sel.w);
                 ra = mma4(px.x, px.y, b0, b1, ra);
+                rm = mma4(px.x, px.y, b0 & KEPT, b1 & KEPT, rm);
                 ra = mma4(px.z, px.w, b2, b3, ra);
-                // ---- mask bits 4i .. 4i+3 and 16+4i .. 16+4i+3: accumulate x over kept rows
-                const uint32_t ms = m >> (4 * i);
-                const u32x4 pm = *reinterpret_cast<const u32x4*>(xw + 32 + hb * 16 + i * 4);
-                rm = mma4(pm.x, pm.y, and_or(ms, B0, G10), and_or(ms, B1, G9), rm);
-                rm = mma4(pm.z, pm.w, and_or(ms, B2, G8), and_or(ms, B3, G7), rm);
+                rm = mma4(px.z, px.w, b2 & KEPT, b3 & KEPT, rm);
             }
             accA[c] = ra;
             accM[c] = rm;
@@ -380,12 +382,13 @@ void matvec_kernel(MatvecArgs a) {
     // staged states (64 halves per unit) then per-unit {sum x, sum off*x}; the
     // same memory is reused for the final reduction
     extern __shared__ __attribute__((aligned(16))) char smem[];
-    h16* xs = reinterpret_cast<h16*>(smem);
-    float* sums = reinterpret_cast<float*>(smem + (size_t)a.units_per_wg * Fmt<BITS, SPARSE>::XS);
-    float* red = reinterpret_cast<float*>(smem);
-    // 16:32 only: table of v_perm selectors per mask byte, behind the sums (the final
-    // reduction reuses the front of the buffer, which never reaches the table)
-    u32x4* lut = reinterpret_cast<u32x4*>(smem + (((size_t)a.units_per_wg * (Fmt<BITS, SPARSE>::XS + 8) + 15) & ~(size_t)15));
+    // 16:32 only: the table of v_perm selectors per mask byte comes first (LDS address
+    // 0: a table index is then a shift of the mask byte and nothing else)
+    constexpr size_t LUT_BYTES = SPARSE ? SPARSE_LUT_BYTES : 0;
+    u32x4* lut = reinterpret_cast<u32x4*>(smem);
+    h16* xs = reinterpret_cast<h16*>(smem + LUT_BYTES);
+    float* sums = reinterpret_cast<float*>(smem + LUT_BYTES + (size_t)a.units_per_wg * Fmt<BITS, SPARSE>::XS);
+    float* red = reinterpret_cast<float*>(smem + LUT_BYTES);
 
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6, nwaves = blockDim.x >> 6;
     const int cl = lane % LC, kl = lane / LC;
@@ -443,7 +446,7 @@ void matvec_kernel(MatvecArgs a) {
             u32x4 e;
 #pragma unroll
             for (int j = 0; j < 4; ++j) e[j] = selb[j] | (0x0Cu << 8) | (selb[j + 4] << 16) | (0x0Cu << 24);
-            lut[b] = e;
+            lut[((b & 15) << 4) | (b >> 4)] = e;                    // stored under the nibble-swapped byte
         }
     }
     if constexpr (FAST) {
@@ -455,8 +458,7 @@ void matvec_kernel(MatvecArgs a) {
                     uint32_t d[16];                                                // d[j] = {x_2j, x_2j+1}
 #pragma unroll
                     for (int i = 0; i < 4; ++i) { d[4 * i] = xv[i].x; d[4 * i + 1] = xv[i].y; d[4 * i + 2] = xv[i].z; d[4 * i + 3] = xv[i].w; }
-                    uint32_t* dstA = reinterpret_cast<uint32_t*>(xs) + (r >> 1) * 64 + (r & 1) * 16;
-                    uint32_t* dstM = dstA + 32;
+                    uint32_t* dstA = reinterpret_cast<uint32_t*>(xs) + r * 16;
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {                                  // rows 8i..8i+7: {x_j, x_j+4}
                         u32x4 p;
@@ -466,22 +468,7 @@ void matvec_kernel(MatvecArgs a) {
                         p.w = __builtin_amdgcn_perm(d[4 * i + 3], d[4 * i + 1], 0x07060302u);
                         *reinterpret_cast<u32x4*>(dstA + 4 * i) = p;
                     }
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) {                                  // {x_p, x_p+16}, p = 4i..4i+3
-                        u32x4 p;
-                        p.x = __builtin_amdgcn_perm(d[8 + 2 * i], d[2 * i], 0x05040100u);
-                        p.y = __builtin_amdgcn_perm(d[8 + 2 * i], d[2 * i], 0x07060302u);
-                        p.z = __builtin_amdgcn_perm(d[9 + 2 * i], d[2 * i + 1], 0x05040100u);
-                        p.w = __builtin_amdgcn_perm(d[9 + 2 * i], d[2 * i + 1], 0x07060302u);
-                        *reinterpret_cast<u32x4*>(dstM + 4 * i) = p;
-                    }
-                    // s: offset of the code part (1024 for every row); o: offset of the mask part
-#pragma unroll
-                    for (int j = 0; j < 16; ++j) {
-                        const float lo = lo_f32(d[j]), hi = hi_f32(d[j]);
-                        s += 1024.f * (lo + hi);
-                        o += lo * (float)(1024 >> ((2 * j) & 3)) + hi * (float)(1024 >> ((2 * j + 1) & 3));
-                    }
+                    // (no magic offsets in this format: the per-unit sums stay 0)
                 } else if constexpr (BITS == 4) {
                     const u32x4 v = xv[0];                                         // x0x1 x2x3 x4x5 x6x7
                     u32x4 p;
@@ -560,12 +547,12 @@ void matvec_kernel(MatvecArgs a) {
 #pragma unroll
             for (int c = 0; c < 4; ++c) { accA[c] = f32x4{0.f, 0.f, 0.f, 0.f}; accM[c] = f32x4{0.f, 0.f, 0.f, 0.f}; }
             const int lu = unit - wg_u0;
-            unit_fast_sparse(un, xs + lu * (Fmt<BITS, SPARSE>::XS / 2), lut, accA, accM);
-            const float offA = sums[lu * 2], offM = sums[lu * 2 + 1];
+            unit_fast_sparse(un, xs + lu * (Fmt<BITS, SPARSE>::XS / 2), reinterpret_cast<const char*>(lut), accA, accM);
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
                 const float sl = fmaxf(sc[c], 0.f);
-                y[c] += sl * ((accA[c][0] - offA) - ze[c] * (accM[c][0] - offM));
+                // A = 2^24 (accA - accM), M = 2^20 accM
+                y[c] += sl * (16777216.f * (accA[c][0] - accM[c][0]) - ze[c] * (1048576.f * accM[c][0]));
                 need_general |= expo[c];
             }
         } else if constexpr (FAST) {
@@ -711,8 +698,8 @@ void matvec_kernel(MatvecArgs a) {
 template <int BITS, bool SPARSE>
 static void launch(const MatvecArgs& a, int lk, bool pf, dim3 grid, dim3 block, hipStream_t st) {
     size_t lds = (size_t)a.units_per_wg * (Fmt<BITS, SPARSE>::XS + 8);     // staged states + per-unit sums
-    if (SPARSE) lds = ((lds + 15) & ~(size_t)15) + 256 * 16;               // selector table
     if (lds < (size_t)block.x * 16) lds = (size_t)block.x * 16;           // reduction area: 4 floats per thread
+    if (SPARSE) lds += SPARSE_LUT_BYTES;                                   // selector tables, in front
 #define I4_LAUNCH(LK_, PF_) hipLaunchKernelGGL((matvec_kernel<BITS, SPARSE, LK_, PF_>), grid, block, lds, st, a)
     if (lk == 1) { if (pf) I4_LAUNCH(1, true); else I4_LAUNCH(1, false); }
     else if (lk == 2) { if (pf) I4_LAUNCH(2, true); else I4_LAUNCH(2, false); }
