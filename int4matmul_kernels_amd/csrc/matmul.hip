@@ -787,9 +787,9 @@ extern "C" int int4mm_matmul(int bits, void* outs, const void* matrix, const voi
 
     hipStream_t st = (hipStream_t)stream;
     // 2 .. 96 rows in all (batches are contiguous, so they flatten): the HBM-bound few-row kernel
-    if (!sparse_mask && B * M >= 2 && B * M <= 96 && !tuning(TUNE_NO_SKINNY) &&
-        skinny_dense(bits, (h16*)outs, (const uint32_t*)matrix, (const h16*)multiplier, (const h16*)scales,
-                    (const h16*)zeros, B * M, K, S, g, false, st))
+    if (B * M >= 2 && B * M <= 96 && !tuning(TUNE_NO_SKINNY) &&
+        skinny_rows(bits, (h16*)outs, (const uint32_t*)matrix, (const h16*)multiplier, (const h16*)scales,
+                    (const h16*)zeros, B * M, K, S, g, false, st, (const uint32_t*)sparse_mask))
         return check_launch("matmul");
 
     MatmulArgs a;

@@ -1,5 +1,5 @@
 // Few-row product for gfx950: 2 .. 96 rows of states (32 per workgroup) against a dense int4 / int3 / int2
-// weight matrix, HBM-bound like the matvec (every packed word is read once and
+// or 16:32 sparse int4 weight matrix, HBM-bound like the matvec (every packed word is read once and
 // used for all rows).  The reference has no such path: it sends M >= 2 to its
 // 64-row matmul tiles (int4matmul.cpp:27) and M == 1 with B > 1 to one matvec
 // per batch element, re-reading the weights each time (matvec_kernel.cu:346).
@@ -25,6 +25,17 @@
 // its W waves split K; each wave stages the states of its own K range through
 // a private LDS buffer, 64 k at a time, and the partial tiles are summed
 // through LDS at the end -- no exchange between workgroups.
+//
+// 16:32 sparse int4 takes the same kernel.  Every lane group loads the block's
+// mask word and both words of kept codes (the four groups of a wave ask for the
+// same addresses); group h skips the codes of the rows before its eight with a
+// population count of the lower mask bits, and expands its codes to their rows
+// with the v_perm selectors of a 256-entry table in LDS (indexed by the mask
+// byte), in the int4 k order.  No magic numbers here: the bytes 0x1q (bit 4: "this
+// row is kept") become the halves 0x001q, i.e. the fp16 denormals (16 + q) 2^-24,
+// which the matrix core multiplies exactly; a second MFMA on the same operand
+// masked to 0x0010 gives 16 * 2^-24 * (sum of the kept rows' states), and
+//     y[m, n] += s[n] * (2^24 (accA - accM) - z[n] * 2^20 accM).
 #include "common.h"
 
 #include <atomic>
@@ -35,6 +46,7 @@ namespace i4 {
 struct SkinnyArgs {
     h16* outs;
     const uint32_t* matrix;
+    const uint32_t* mask;   // 16:32 sparse only
     const h16* x;
     const h16* scales;
     const h16* zeros;
@@ -74,7 +86,12 @@ __device__ __forceinline__ uint32_t vgpr_const(uint32_t literal) {
 // the packed rows of a 32-row block.
 //   int4: order 0,4,1,5,2,6,3,7; registers 0, 2 carry 1024 + q, registers 1, 3 carry 64 + q
 //   int2: natural order, {1024 + q_even, 256 + q_odd};  int3: natural order, {1024 + q_even, 128 + q_odd}
-template <int BITS> struct SkFmt;
+template <int BITS, bool SPARSE = false> struct SkFmt;
+template <> struct SkFmt<4, true> {
+    static constexpr int ROWS = 2, LOADS = 6;            // per block: two words of codes and the mask word
+    __device__ static constexpr int order(int e) { return (e >> 1) + 4 * (e & 1); }
+    __device__ static constexpr uint32_t offs(int) { return 0u; }
+};
 template <> struct SkFmt<4> {
     static constexpr int ROWS = 4, LOADS = 2;            // packed rows per block, loads per lane and unit
     __device__ static constexpr int order(int e) { return (e >> 1) + 4 * (e & 1); }
@@ -110,6 +127,27 @@ __device__ __forceinline__ h16x8 magic_operand(uint32_t f, uint32_t m0, uint32_t
     return bitcast<h16x8>(r);
 }
 
+// 16:32: `v` = the chunk's kept codes as consecutive nibbles, `sel` = the selectors of its mask byte
+__device__ __forceinline__ u32x4 sparse_operand(uint32_t v, const u32x4& sel, uint32_t nib, uint32_t flag) {
+    const uint32_t even = (v & nib) | flag, odd = ((v >> 4) & nib) | flag;
+    return u32x4{__builtin_amdgcn_perm(odd, even, sel.x), __builtin_amdgcn_perm(odd, even, sel.y),
+                 __builtin_amdgcn_perm(odd, even, sel.z), __builtin_amdgcn_perm(odd, even, sel.w)};
+}
+
+__device__ __forceinline__ h16x8 exact_operand_sparse(uint32_t v, uint32_t m8, h16 sc, h16 ze) {
+    h16 row[8];
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+        const bool kept = (m8 >> r) & 1u;
+        row[r] = kept ? dequant_code<4>(v & 15u, sc, ze) : (h16)0.0f;
+        v >>= kept ? 4 : 0;
+    }
+    h16x8 o;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) o[e] = row[SkFmt<4, true>::order(e)];
+    return o;
+}
+
 template <int BITS>
 __device__ __forceinline__ h16x8 exact_operand(uint32_t f, h16 sc, h16 ze) {
     h16x8 r;
@@ -121,11 +159,11 @@ __device__ __forceinline__ h16x8 exact_operand(uint32_t f, h16 sc, h16 ze) {
 
 // CW: columns per lane; RT: row groups of 8 that can hold real rows (R <= 8 RT);
 // MT: 16-row MFMA tiles; PF: units of packed weights in flight per wave
-template <int BITS, int CW, int RT>
+template <int BITS, int CW, int RT, bool SPARSE>
 __global__ __launch_bounds__(512) void skinny_kernel(SkinnyArgs a) {
-    using F = SkFmt<BITS>;
+    using F = SkFmt<BITS, SPARSE>;
     constexpr int NL = F::LOADS;
-    constexpr int PF = BITS == 3 && CW == 4 ? 2 : 4, MT = RT == 4 ? 2 : 1;
+    constexpr int PF = (BITS == 3 && CW == 4) || (SPARSE && CW == 4) ? 2 : 4, MT = RT == 4 ? 2 : 1;
     constexpr int PFX = RT == 4 ? 2 : 4;            // units of states in flight per wave
     constexpr int STRIP = 16 * CW;
     extern __shared__ __attribute__((aligned(16))) char lds[];
@@ -146,7 +184,29 @@ __global__ __launch_bounds__(512) void skinny_kernel(SkinnyArgs a) {
     // strip switch the whole workgroup to the exact per-weight decode.  (The copy
     // runs after the first loads have been issued, under their latency.)
     const int groups = (units + a.group_units - 1) / a.group_units;
-    uint32_t* sz = reinterpret_cast<uint32_t*>(lds + nwaves * SK_WAVE_LDS + 16);      // scales, then zeros
+    // (16:32: the selector table sits between the waves' buffers and the scales)
+    constexpr int LUT_BYTES = SPARSE ? 256 * 16 : 0;
+    const char* lut = lds + nwaves * SK_WAVE_LDS + 16;
+    if constexpr (SPARSE) {
+        // for mask byte b, pair e = (row e, row e + 4): byte 0 picks the code byte of row e out of
+        // {even nibbles, odd nibbles} by its rank among the kept rows, byte 2 that of row e + 4;
+        // 0x0C yields 0.  Stored under the nibble-swapped byte (see the lookup).
+        for (int b = t; b < 256; b += blockDim.x) {
+            uint32_t selb[8];
+            int rank = 0;
+#pragma unroll
+            for (int r = 0; r < 8; ++r) {
+                const bool k = (b >> r) & 1;
+                selb[r] = k ? (uint32_t)((rank & 1) * 4 + (rank >> 1)) : 0x0Cu;
+                rank += k;
+            }
+            u32x4 e;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) e[q] = selb[q] | (0x0Cu << 8) | (selb[q + 4] << 16) | (0x0Cu << 24);
+            *reinterpret_cast<u32x4*>(lds + nwaves * SK_WAVE_LDS + 16 + (((b & 15) << 4) | (b >> 4)) * 16) = e;
+        }
+    }
+    uint32_t* sz = reinterpret_cast<uint32_t*>(lds + nwaves * SK_WAVE_LDS + 16 + LUT_BYTES);      // scales, then zeros
     auto scan_scales = [&]() -> bool {
         int* flag = reinterpret_cast<int*>(lds + nwaves * SK_WAVE_LDS);
         if (t == 0) *flag = 0;
@@ -172,11 +232,16 @@ __global__ __launch_bounds__(512) void skinny_kernel(SkinnyArgs a) {
 
     // accumulators: acc = raw products of the current group, y = finished groups
     // (register e of tile mt is row 16 mt + 4 h + e, column j)
-    f32x4 acc[CW][MT], y[CW][MT];
+    // (16:32: accm = the same for the "kept" flags)
+    f32x4 acc[CW][MT], accm[SPARSE ? CW : 1][MT], y[CW][MT];
 #pragma unroll
     for (int c = 0; c < CW; ++c)
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) { acc[c][mt] = f32x4{0.f, 0.f, 0.f, 0.f}; y[c][mt] = f32x4{0.f, 0.f, 0.f, 0.f}; }
+        for (int mt = 0; mt < MT; ++mt) {
+            acc[c][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+            y[c][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+            if (SPARSE || c == 0) accm[SPARSE ? c : 0][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+        }
 
     if (u0 >= u1) general = scan_scales();          // idle waves still take part in its barriers
     if (u0 < u1) {
@@ -188,15 +253,30 @@ __global__ __launch_bounds__(512) void skinny_kernel(SkinnyArgs a) {
         //         next one, shifted right by {0, 24, 16, 40}[h]
         const int wrow = BITS == 4 ? h : (BITS == 2 ? (h >> 1) : (h >> 1));
         const int wshift = BITS == 4 ? 0 : (BITS == 2 ? 16 * (h & 1) : (h == 0 ? 0 : h == 1 ? 24 : h == 2 ? 16 : 40));
-        const uint32_t* wbase = a.matrix + (int64_t)wrow * a.S + col0;
+        //   16:32: every lane group loads both words of kept codes and the mask word of the block
+        //          (w[3 blk], w[3 blk + 1], w[3 blk + 2])
+        const uint32_t* wbase = a.matrix + (int64_t)(SPARSE ? 0 : wrow) * a.S + col0;
+        const uint32_t* mbase = SPARSE ? a.mask + col0 : nullptr;
         auto load_w = [&](words_t w[NL], int u) {
             const uint32_t* p = wbase + (int64_t)u * (2 * F::ROWS) * a.S;
+            if constexpr (SPARSE) {
+                const uint32_t* pm = mbase + (int64_t)u * 2 * a.S;
 #pragma unroll
-            for (int i = 0; i < NL; ++i) {
-                const int row = BITS == 3 ? 3 * (i >> 1) + (i & 1) : F::ROWS * i;       // relative to the lane's first row
-                w[i] = __builtin_nontemporal_load(reinterpret_cast<const words_t*>(p + (int64_t)row * a.S));
+                for (int blk = 0; blk < 2; ++blk) {
+                    w[3 * blk] = __builtin_nontemporal_load(reinterpret_cast<const words_t*>(p + (int64_t)(2 * blk) * a.S));
+                    w[3 * blk + 1] = __builtin_nontemporal_load(reinterpret_cast<const words_t*>(p + (int64_t)(2 * blk + 1) * a.S));
+                    w[3 * blk + 2] = __builtin_nontemporal_load(reinterpret_cast<const words_t*>(pm + (int64_t)blk * a.S));
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < NL; ++i) {
+                    const int row = BITS == 3 ? 3 * (i >> 1) + (i & 1) : F::ROWS * i;       // relative to the lane's first row
+                    w[i] = __builtin_nontemporal_load(reinterpret_cast<const words_t*>(p + (int64_t)row * a.S));
+                }
             }
         };
+        // 16:32: mask bits of the rows before the lane group's eight; selector that replicates mask byte h
+        const uint32_t below = SPARSE ? (1u << (8 * h)) - 1u : 0u, rep_h = 0x01010101u * h;
         // the 8 codes of chunk h of block blk, column c
         auto chunk_bits = [&](const words_t w[NL], int blk, int c) -> uint32_t {
             if constexpr (BITS == 3)
@@ -248,6 +328,8 @@ __global__ __launch_bounds__(512) void skinny_kernel(SkinnyArgs a) {
         const uint32_t m0 = vgpr_const(BITS == 4 ? 0x000F000Fu : BITS == 2 ? 0x000C0003u : 0x00380007u);
         const uint32_t g0 = vgpr_const(BITS == 4 ? 0x64006400u : BITS == 2 ? 0x5C006400u : 0x58006400u);
         const uint32_t m1 = BITS == 4 ? vgpr_const(0x00F000F0u) : 0u, g1 = BITS == 4 ? vgpr_const(0x54005400u) : 0u;
+        const uint32_t sp_nib = SPARSE ? vgpr_const(0x0F0F0F0Fu) : 0u, sp_flag = SPARSE ? vgpr_const(0x10101010u) : 0u;
+        const uint32_t sp_kept = SPARSE ? vgpr_const(0x00100010u) : 0u, sp_idx = SPARSE ? vgpr_const(0x00000FF0u) : 0u;
         float gS = 0.f, gO = 0.f;           // sums of the current group so far (row lane / 2)
         float nS, nO;                       // sums of the unit staged last (the next to be multiplied)
         // scale / zero of the lane's CW columns for group gi, from the LDS copy
@@ -295,12 +377,37 @@ __global__ __launch_bounds__(512) void skinny_kernel(SkinnyArgs a) {
                     xa[mt] = *reinterpret_cast<const h16x8*>(my + p * SK_XBUF + (j + 16 * mt) * SK_PITCH + (i * 4 + h) * 16);
 #pragma unroll
                 for (int c = 0; c < CW; ++c) {
-                    const uint32_t f = chunk_bits(w, i, c);
-                    const h16x8 wb = general ? exact_operand<BITS>(f, sc[c], ze[c])
-                                             : magic_operand<BITS>(f, m0, m1, g0, g1);
+                    if constexpr (SPARSE) {
+                        const uint32_t m = word_of<CW>(w[3 * i + 2], c);
+                        const uint64_t st = ((uint64_t)word_of<CW>(w[3 * i + 1], c) << 32) | word_of<CW>(w[3 * i], c);
+                        // the codes of the rows before this chunk are skipped, 4 bits each (a full
+                        // skip of 64 bits only happens when no row of the chunk is kept)
+                        const uint32_t v = (uint32_t)(st >> ((uint32_t)__builtin_popcount(m & below) << 2));
+                        const uint32_t mb4 = __builtin_amdgcn_perm(m, m, rep_h);           // mask byte h, four times
+                        if constexpr (general) {
+                            const h16x8 wb = exact_operand_sparse(v, mb4 & 0xFFu, sc[c], ze[c]);
 #pragma unroll
-                    for (int mt = 0; mt < MT; ++mt)
-                        acc[c][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[mt], wb, acc[c][mt], 0, 0, 0);
+                            for (int mt = 0; mt < MT; ++mt)
+                                acc[c][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[mt], wb, acc[c][mt], 0, 0, 0);
+                        } else {
+                            // (table entries sit under the nibble-swapped byte = bits 4 .. 11 of mb4)
+                            const u32x4 sel = *reinterpret_cast<const u32x4*>(lut + (mb4 & sp_idx));
+                            const u32x4 b = sparse_operand(v, sel, sp_nib, sp_flag);
+                            const u32x4 bm = u32x4{b.x & sp_kept, b.y & sp_kept, b.z & sp_kept, b.w & sp_kept};
+#pragma unroll
+                            for (int mt = 0; mt < MT; ++mt) {
+                                acc[c][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[mt], bitcast<h16x8>(b), acc[c][mt], 0, 0, 0);
+                                accm[c][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[mt], bitcast<h16x8>(bm), accm[c][mt], 0, 0, 0);
+                            }
+                        }
+                    } else {
+                        const uint32_t f = chunk_bits(w, i, c);
+                        const h16x8 wb = general ? exact_operand<BITS>(f, sc[c], ze[c])
+                                                 : magic_operand<BITS>(f, m0, m1, g0, g1);
+#pragma unroll
+                        for (int mt = 0; mt < MT; ++mt)
+                            acc[c][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[mt], wb, acc[c][mt], 0, 0, 0);
+                    }
                 }
             }
             // refill this register set PF units ahead; move the next unit's states to LDS
@@ -321,10 +428,16 @@ __global__ __launch_bounds__(512) void skinny_kernel(SkinnyArgs a) {
                         const float z = general ? 0.f : (float)ze[c];
 #pragma unroll
                         for (int e = 0; e < 4; ++e) {
-                            const float off = general ? 0.f : o4[e] + z * s4[e];
-                            y[c][mt][e] += sf * (acc[c][mt][e] - off);
+                            if constexpr (SPARSE && !general) {
+                                // A = 2^24 (acc - accm), sum of the kept rows' states = 2^20 accm
+                                y[c][mt][e] += sf * (16777216.f * (acc[c][mt][e] - accm[c][mt][e]) - z * (1048576.f * accm[c][mt][e]));
+                            } else {
+                                const float off = general ? 0.f : o4[e] + z * s4[e];
+                                y[c][mt][e] += sf * (acc[c][mt][e] - off);
+                            }
                         }
                         acc[c][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+                        if constexpr (SPARSE) accm[c][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
                     }
                 }
                 gS = 0.f; gO = 0.f;
@@ -390,12 +503,12 @@ __global__ __launch_bounds__(512) void skinny_kernel(SkinnyArgs a) {
     }
 }
 
-template <int BITS, int CW>
+template <int BITS, int CW, bool SPARSE>
 static bool launch_skinny(const SkinnyArgs& a, int waves, hipStream_t st) {
     const int strips = a.S / (16 * CW);
     const int rt = ((a.R > 32 ? 32 : a.R) + 7) / 8;
     const int groups = (a.K / 64 + a.group_units - 1) / a.group_units;
-    size_t lds = (size_t)waves * SK_WAVE_LDS + 16 + (size_t)groups * 16 * CW * 4;
+    size_t lds = (size_t)waves * SK_WAVE_LDS + 16 + (SPARSE ? 256 * 16 : 0) + (size_t)groups * 16 * CW * 4;
     const size_t red = (size_t)(waves / 2) * (rt <= 2 ? 1 : 2) * 16 * 16 * CW * 4;
     if (red > lds) lds = red;
     if (lds > 150 * 1024) return false;
@@ -413,43 +526,49 @@ static bool launch_skinny(const SkinnyArgs& a, int waves, hipStream_t st) {
         }
         hipLaunchKernelGGL(kernel, grid, block, lds, st, a);
     };
-    if (rt <= 1) go(skinny_kernel<BITS, CW, 1>, 0);
-    else if (rt <= 2) go(skinny_kernel<BITS, CW, 2>, 1);
-    else go(skinny_kernel<BITS, CW, 4>, 2);
+    if (rt <= 1) go(skinny_kernel<BITS, CW, 1, SPARSE>, 0);
+    else if (rt <= 2) go(skinny_kernel<BITS, CW, 2, SPARSE>, 1);
+    else go(skinny_kernel<BITS, CW, 4, SPARSE>, 2);
     return true;
 }
 
-template <int BITS>
+template <int BITS, bool SPARSE = false>
 static bool launch_skinny_cw(const SkinnyArgs& a, int cw, int waves, hipStream_t st) {
-    if (cw == 4) return launch_skinny<BITS, 4>(a, waves, st);
-    if (cw == 2) return launch_skinny<BITS, 2>(a, waves, st);
-    return launch_skinny<BITS, 1>(a, waves, st);
+    if (cw == 4) return launch_skinny<BITS, 4, SPARSE>(a, waves, st);
+    if (cw == 2) return launch_skinny<BITS, 2, SPARSE>(a, waves, st);
+    return launch_skinny<BITS, 1, SPARSE>(a, waves, st);
 }
 
-// Product of R <= 96 rows with a dense matrix (beyond that the tile kernels are faster).  Returns false when the shape is
-// not one this kernel takes (the caller then uses the general kernels).
-bool skinny_dense(int bits, h16* outs, const uint32_t* matrix, const h16* x, const h16* scales, const h16* zeros,
-                 int64_t R, int64_t K, int64_t S, int64_t group_size, bool accumulate, hipStream_t st) {
+// Product of 2 <= R <= 96 rows with a dense or (sparse_mask != nullptr) 16:32 sparse int4 matrix; beyond that
+// the tile kernels are faster.  Returns false when the shape is not one this kernel takes (the caller then
+// uses the general kernels).
+bool skinny_rows(int bits, h16* outs, const uint32_t* matrix, const h16* x, const h16* scales, const h16* zeros,
+                 int64_t R, int64_t K, int64_t S, int64_t group_size, bool accumulate, hipStream_t st,
+                 const uint32_t* sparse_mask) {
     if (R < 2 || R > 96 || S % 16 != 0 || K % 64 != 0 || K > (1 << 30) || S > (1 << 28)) return false;
+    if (sparse_mask && bits != 4) return false;
     SkinnyArgs a;
-    a.outs = outs; a.matrix = matrix; a.x = x; a.scales = scales; a.zeros = zeros;
+    a.outs = outs; a.matrix = matrix; a.mask = sparse_mask; a.x = x; a.scales = scales; a.zeros = zeros;
     a.R = (int)R; a.K = (int)K; a.S = (int)S;
     const int64_t gu = group_size / 64;
     a.group_units = (int)(gu > 0x7FFFFFF ? 0x7FFFFFF : gu);
     a.accumulate = accumulate ? 1 : 0;
     // widest strips (64, 32 or 16 columns) that still give at least 256 workgroups,
     // else at least 128 (narrow strips use half a cache line per packed row);
-    // four waves split K when there are 256 workgroups (three of them fit a CU),
-    // eight otherwise
+    // four waves split K when there are 256 workgroups (three of them fit a CU) and K
+    // is short (each wave should walk a dozen units or more), eight otherwise
     int cw = 1;
     const int prefer[4][2] = {{4, 256}, {2, 256}, {4, 128}, {2, 128}};       // {columns per lane, workgroups}
     for (const auto& c : prefer)
         if (S % (16 * c[0]) == 0 && S / (16 * c[0]) >= c[1]) { cw = c[0]; break; }
+    // (16:32 with more than 16 rows: four columns per lane would not fit the register file)
+    if (sparse_mask && R > 16 && cw == 4) cw = 2;
     const int units = (int)(K / 64);
     int waves = (int)tuning(TUNE_MV_WAVES);
-    if (waves != 2 && waves != 4 && waves != 8) waves = S / (16 * cw) >= 256 ? 4 : 8;
+    if (waves != 2 && waves != 4 && waves != 8) waves = S / (16 * cw) >= 256 && units < 160 ? 4 : 8;
     while (waves > 1 && units < 2 * waves) waves >>= 1;
     a.units_per_wave = (units + waves - 1) / waves;
+    if (sparse_mask) return launch_skinny_cw<4, true>(a, cw, waves, st);
     if (bits == 4) return launch_skinny_cw<4>(a, cw, waves, st);
     if (bits == 3) return launch_skinny_cw<3>(a, cw, waves, st);
     return launch_skinny_cw<2>(a, cw, waves, st);

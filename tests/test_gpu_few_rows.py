@@ -1,5 +1,5 @@
-"""The few-row kernel (2 .. 96 rows of states in all, dense formats): every packed
-word is read once for all rows.  It serves `quant_matmul` with small M (any
+"""The few-row kernel (2 .. 96 rows of states in all; dense formats and 16:32
+sparse int4): every packed word is read once for all rows.  It serves `quant_matmul` with small M (any
 batch layout that flattens to <= 32 rows) and the matvec entry with B > 1.
 Its numerics are the matvec's (exact sum of x (q - z) s, no per-weight fp16
 rounding), so the matvec tolerance applies; it is also checked against the
@@ -84,4 +84,81 @@ def test_few_rows_degenerate_known_answer(H, bits):
 def test_few_rows_full_size(H, bits):
     """K=5120, S=20480, 16 rows: the whole output against the oracle"""
     p = _problem(bits, K=5120, S=20480, M=16, group_size=128, seed=4)
+    _check(H, p, "mtx")
+
+
+# ---- 16:32 sparse int4 through the same kernel
+@pytest.mark.parametrize("M", [2, 3, 8, 9, 16, 17, 32, 33, 64, 96])
+@pytest.mark.parametrize("K,S,g", [(512, 256, 64), (64, 64, 64), (1024, 192, -1), (320, 1024, 64), (256, 8192, 128)])
+def test_few_rows_sparse_matmul(H, M, K, S, g):
+    p = O.make_problem(bits=4, K=K, S=S, M=M, group_size=g, sparse=True, seed=M + K)
+    junk = np.full((1, M, S), -77.0, np.float16)
+    d, got = _check(H, p, "mtx", prior=junk)
+    H.capi.tune(5, 1)
+    try:
+        ref = H.run_capi(p, d, "mtx")
+    finally:
+        H.capi.tune(5, 0)
+    assert O.max_rel_error(ref.astype(np.float64), got) < H.TOL_EXACT
+
+
+@pytest.mark.parametrize("B,M", [(2, 1), (5, 1), (32, 1), (4, 4), (3, 7), (40, 1), (96, 1)])
+def test_few_rows_sparse_batches_flatten(H, B, M):
+    p = O.make_problem(bits=4, K=768, S=320, M=M, group_size=64, sparse=True, seed=B * 10 + M, B=B)
+    _check(H, p, "mtx")
+    if M == 1:
+        prior = np.random.default_rng(B).standard_normal((B, 1, 320)).astype(np.float16)
+        _check(H, p, "vec", prior=prior)
+
+
+def test_few_rows_sparse_exponent_mode_columns(H):
+    p = O.make_problem(bits=4, K=512, S=256, M=6, group_size=64, sparse=True, seed=9)
+    p["scales"][1, 40:48] *= np.float16(-1)
+    p["scales"][3, 200] *= np.float16(-1)
+    _check(H, p, "mtx")
+
+
+def test_few_rows_sparse_crowded_masks(H):
+    """masks whose kept rows crowd one end of the block: all 16 codes lie before, or
+    after, some 8-row chunk"""
+    K, S, M = 256, 64, 5
+    rng = np.random.default_rng(3)
+    codes = rng.integers(0, 16, size=(K, S), dtype=np.uint8)
+    keep = np.zeros((K // 32, 32, S), dtype=bool)
+    keep[0, :16] = True                      # first half
+    keep[1, 16:] = True                      # second half
+    keep[2, 8:24] = True                     # the middle
+    keep[3, ::2] = True                      # every other row
+    keep[4, :8] = True
+    keep[4, 24:] = True                      # both ends
+    keep[5, 1::2] = True
+    keep[6, :4] = True
+    keep[6, 20:] = True
+    keep[7, 3:19] = True
+    keep = keep.reshape(K, S)
+    matrix, mask = O.sparse_pack(np.ascontiguousarray(codes.T), np.ascontiguousarray(keep.T).astype(np.uint8))
+    G = K // 64
+    p = dict(B=1, M=M, S=S, K=K, bits=4, group_size=64, matrix=matrix, sparse_mask=mask, keep=keep,
+             codes=np.where(keep, codes, np.uint8(0)), states=rng.standard_normal((1, M, K)).astype(np.float16),
+             scales=rng.uniform(0.001, 0.02, size=(G, S)).astype(np.float16),
+             zeros=rng.uniform(0, 15, size=(G, S)).astype(np.float16))
+    _check(H, p, "mtx")
+    _check(H, dict(p, M=1, states=p["states"][:, :1]), "vec")
+
+
+def test_few_rows_sparse_degenerate_known_answer(H):
+    K, S, M = 1024, 128, 12
+    codes = np.ones((S, K), np.uint8)
+    keep = np.zeros((S, K), np.uint8)
+    keep[:, ::2] = 1
+    matrix, mask = O.sparse_pack(codes, keep)
+    p = dict(B=1, M=M, S=S, K=K, bits=4, group_size=64, matrix=matrix, sparse_mask=mask,
+             states=np.ones((1, M, K), np.float16), scales=np.ones((K // 64, S), np.float16),
+             zeros=np.zeros((K // 64, S), np.float16))
+    got = H.run_capi(p, H.dev_problem(p), "mtx")
+    assert np.all(got.astype(np.float64) == K // 2)
+
+
+def test_few_rows_sparse_full_size(H):
+    p = O.make_problem(bits=4, K=5120, S=20480, M=8, group_size=64, sparse=True, seed=4)
     _check(H, p, "mtx")
