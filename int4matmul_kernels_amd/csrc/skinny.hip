@@ -307,18 +307,22 @@ __global__ __launch_bounds__(512) void skinny_kernel(SkinnyArgs a) {
                 if constexpr (BITS == 4)
                     q = u32x4{__builtin_amdgcn_perm(v[2], v[0], 0x05040100u), __builtin_amdgcn_perm(v[2], v[0], 0x07060302u),
                               __builtin_amdgcn_perm(v[3], v[1], 0x05040100u), __builtin_amdgcn_perm(v[3], v[1], 0x07060302u)};
+                if constexpr (!SPARSE) {                 // (16:32 has no offsets to remove)
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    sx = dot2(q[e], ONES, sx);
-                    so = dot2(q[e], F::offs(e), so);
+                    for (int e = 0; e < 4; ++e) {
+                        sx = dot2(q[e], ONES, sx);
+                        so = dot2(q[e], F::offs(e), so);
+                    }
                 }
                 *reinterpret_cast<u32x4*>(my + p * SK_XBUF + xm * SK_PITCH + (xpart * RT + i) * 16) = q;
             }
-            // the other lanes of the row: lane ^ 1, lane ^ 2, lane ^ 4 as far as the row extends
-            sx += dpp_f32<0xB1>(sx);
-            so += dpp_f32<0xB1>(so);
-            if constexpr (LPR >= 4) { sx += dpp_f32<0x4E>(sx); so += dpp_f32<0x4E>(so); }
-            if constexpr (LPR >= 8) { sx += dpp_f32<0x141>(sx); so += dpp_f32<0x141>(so); }
+            if constexpr (!SPARSE) {
+                // the other lanes of the row: lane ^ 1, lane ^ 2, lane ^ 4 as far as the row extends
+                sx += dpp_f32<0xB1>(sx);
+                so += dpp_f32<0xB1>(so);
+                if constexpr (LPR >= 4) { sx += dpp_f32<0x4E>(sx); so += dpp_f32<0x4E>(so); }
+                if constexpr (LPR >= 8) { sx += dpp_f32<0x141>(sx); so += dpp_f32<0x141>(so); }
+            }
         };
         // rows that never receive states must read as zero
         for (int i = lane; i < 2 * SK_XBUF / 16; i += 64) *reinterpret_cast<u32x4*>(my + i * 16) = u32x4{0, 0, 0, 0};
@@ -416,6 +420,23 @@ __global__ __launch_bounds__(512) void skinny_kernel(SkinnyArgs a) {
             load_x(xn, min(u + 1 + PFX, u1 - 1));
             // group complete (or this wave's range ends): fold it into y
             if ((u + 1) % a.group_units == 0 || u + 1 == u1) {
+                if constexpr (SPARSE && !general) {
+                    load_sz(u / a.group_units);
+#pragma unroll
+                    for (int c = 0; c < CW; ++c) {
+                        // y += s (A - z M) with A = 2^24 (acc - accm), M = 2^20 accm
+                        const float ka = (float)sc[c] * 16777216.f;
+                        const float km = -(ka + (float)sc[c] * (float)ze[c] * 1048576.f);
+#pragma unroll
+                        for (int mt = 0; mt < MT; ++mt) {
+#pragma unroll
+                            for (int e = 0; e < 4; ++e)
+                                y[c][mt][e] = __builtin_fmaf(ka, acc[c][mt][e], __builtin_fmaf(km, accm[c][mt][e], y[c][mt][e]));
+                            acc[c][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+                            accm[c][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+                        }
+                    }
+                } else {
                 if (xpart == 0) { sums[xm] = gS; sums[32 + xm] = gO; }
                 if constexpr (!general) load_sz(u / a.group_units);
 #pragma unroll
@@ -428,17 +449,12 @@ __global__ __launch_bounds__(512) void skinny_kernel(SkinnyArgs a) {
                         const float z = general ? 0.f : (float)ze[c];
 #pragma unroll
                         for (int e = 0; e < 4; ++e) {
-                            if constexpr (SPARSE && !general) {
-                                // A = 2^24 (acc - accm), sum of the kept rows' states = 2^20 accm
-                                y[c][mt][e] += sf * (16777216.f * (acc[c][mt][e] - accm[c][mt][e]) - z * (1048576.f * accm[c][mt][e]));
-                            } else {
-                                const float off = general ? 0.f : o4[e] + z * s4[e];
-                                y[c][mt][e] += sf * (acc[c][mt][e] - off);
-                            }
+                            const float off = general ? 0.f : o4[e] + z * s4[e];
+                            y[c][mt][e] += sf * (acc[c][mt][e] - off);
                         }
                         acc[c][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
-                        if constexpr (SPARSE) accm[c][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
                     }
+                }
                 }
                 gS = 0.f; gO = 0.f;
             }
