@@ -245,7 +245,6 @@ __host__ __device__ constexpr uint32_t pair_selector(int a, int b) {
 // bits 4..11 are the table offset (entries are stored under the nibble-swapped byte).
 // Staged states per unit: for each block 16 dwords {x_j, x_j+4}, ordered as the
 // dense int4 path.
-constexpr int SPARSE_LUT_BYTES = 256 * 16;
 
 __device__ __forceinline__ void unit_fast_sparse(const Unit<4, true>& u, const h16* xp, const char* lut,
                                                  f32x4 accA[4], f32x4 accM[4]) {
@@ -382,13 +381,12 @@ void matvec_kernel(MatvecArgs a) {
     // staged states (64 halves per unit) then per-unit {sum x, sum off*x}; the
     // same memory is reused for the final reduction
     extern __shared__ __attribute__((aligned(16))) char smem[];
-    // 16:32 only: the table of v_perm selectors per mask byte comes first (LDS address
-    // 0: a table index is then a shift of the mask byte and nothing else)
-    constexpr size_t LUT_BYTES = SPARSE ? SPARSE_LUT_BYTES : 0;
-    u32x4* lut = reinterpret_cast<u32x4*>(smem);
-    h16* xs = reinterpret_cast<h16*>(smem + LUT_BYTES);
-    float* sums = reinterpret_cast<float*>(smem + LUT_BYTES + (size_t)a.units_per_wg * Fmt<BITS, SPARSE>::XS);
-    float* red = reinterpret_cast<float*>(smem + LUT_BYTES);
+    // 16:32 only: the table of v_perm selectors per mask byte, statically allocated so that
+    // its LDS address is a compile-time constant (a table read then needs no address add)
+    __shared__ __attribute__((aligned(16))) u32x4 lut[SPARSE ? 256 : 1];
+    h16* xs = reinterpret_cast<h16*>(smem);
+    float* sums = reinterpret_cast<float*>(smem + (size_t)a.units_per_wg * Fmt<BITS, SPARSE>::XS);
+    float* red = reinterpret_cast<float*>(smem);
 
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6, nwaves = blockDim.x >> 6;
     const int cl = lane % LC, kl = lane / LC;
@@ -699,7 +697,6 @@ template <int BITS, bool SPARSE>
 static void launch(const MatvecArgs& a, int lk, bool pf, dim3 grid, dim3 block, hipStream_t st) {
     size_t lds = (size_t)a.units_per_wg * (Fmt<BITS, SPARSE>::XS + 8);     // staged states + per-unit sums
     if (lds < (size_t)block.x * 16) lds = (size_t)block.x * 16;           // reduction area: 4 floats per thread
-    if (SPARSE) lds += SPARSE_LUT_BYTES;                                   // selector tables, in front
 #define I4_LAUNCH(LK_, PF_) hipLaunchKernelGGL((matvec_kernel<BITS, SPARSE, LK_, PF_>), grid, block, lds, st, a)
     if (lk == 1) { if (pf) I4_LAUNCH(1, true); else I4_LAUNCH(1, false); }
     else if (lk == 2) { if (pf) I4_LAUNCH(2, true); else I4_LAUNCH(2, false); }

@@ -184,9 +184,9 @@ __global__ __launch_bounds__(512) void skinny_kernel(SkinnyArgs a) {
     // strip switch the whole workgroup to the exact per-weight decode.  (The copy
     // runs after the first loads have been issued, under their latency.)
     const int groups = (units + a.group_units - 1) / a.group_units;
-    // (16:32: the selector table sits between the waves' buffers and the scales)
-    constexpr int LUT_BYTES = SPARSE ? 256 * 16 : 0;
-    const char* lut = lds + nwaves * SK_WAVE_LDS + 16;
+    // (16:32: the selector table is allocated statically: its LDS address is a compile-time constant)
+    __shared__ __attribute__((aligned(16))) u32x4 lut_table[SPARSE ? 256 : 1];
+    const char* lut = reinterpret_cast<const char*>(lut_table);
     if constexpr (SPARSE) {
         // for mask byte b, pair e = (row e, row e + 4): byte 0 picks the code byte of row e out of
         // {even nibbles, odd nibbles} by its rank among the kept rows, byte 2 that of row e + 4;
@@ -203,10 +203,10 @@ __global__ __launch_bounds__(512) void skinny_kernel(SkinnyArgs a) {
             u32x4 e;
 #pragma unroll
             for (int q = 0; q < 4; ++q) e[q] = selb[q] | (0x0Cu << 8) | (selb[q + 4] << 16) | (0x0Cu << 24);
-            *reinterpret_cast<u32x4*>(lds + nwaves * SK_WAVE_LDS + 16 + (((b & 15) << 4) | (b >> 4)) * 16) = e;
+            lut_table[((b & 15) << 4) | (b >> 4)] = e;
         }
     }
-    uint32_t* sz = reinterpret_cast<uint32_t*>(lds + nwaves * SK_WAVE_LDS + 16 + LUT_BYTES);      // scales, then zeros
+    uint32_t* sz = reinterpret_cast<uint32_t*>(lds + nwaves * SK_WAVE_LDS + 16);      // scales, then zeros
     auto scan_scales = [&]() -> bool {
         int* flag = reinterpret_cast<int*>(lds + nwaves * SK_WAVE_LDS);
         if (t == 0) *flag = 0;
@@ -524,10 +524,10 @@ static bool launch_skinny(const SkinnyArgs& a, int waves, hipStream_t st) {
     const int strips = a.S / (16 * CW);
     const int rt = ((a.R > 32 ? 32 : a.R) + 7) / 8;
     const int groups = (a.K / 64 + a.group_units - 1) / a.group_units;
-    size_t lds = (size_t)waves * SK_WAVE_LDS + 16 + (SPARSE ? 256 * 16 : 0) + (size_t)groups * 16 * CW * 4;
+    size_t lds = (size_t)waves * SK_WAVE_LDS + 16 + (size_t)groups * 16 * CW * 4;
     const size_t red = (size_t)(waves / 2) * (rt <= 2 ? 1 : 2) * 16 * 16 * CW * 4;
     if (red > lds) lds = red;
-    if (lds > 150 * 1024) return false;
+    if (lds > 150 * 1024 - (SPARSE ? 4096 : 0)) return false;      // (16:32: 4 KB of static LDS for the selector table)
     const dim3 grid(strips, (a.R + 31) / 32), block(waves * 64);
     auto go = [&](auto kernel, int slot) {
         // more than 64 KB of dynamic LDS has to be requested once per kernel and device
