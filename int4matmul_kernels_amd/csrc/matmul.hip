@@ -610,21 +610,30 @@ __device__ __forceinline__ void pipe_tile(const MatmulArgs& a, const int m0, con
                     advance_a();
                     advance();
                 }
-                write_b_fast(r_dec, b2, ks);
+                if (ks == 0) { write_b_fast(r_dec, b2, 0); write_b_fast(r_dec, b2, 1); }
                 if (ks == 1) write_a(ra_wr, b2);
                 mfma_slice(fa[ks], fb[ks]);
-                // scheduling template of this k slice: the next slice's fragment reads
-                // first, then every MFMA followed by a few decode instructions (and, in
-                // the first slice, one of this step's global loads), the LDS stores last
-                __builtin_amdgcn_sched_group_barrier(0x100, TM + TN + (SPARSE ? 2 : 0), 0);
+                // scheduling template.  First slice: the next slice's fragment reads, then
+                // every MFMA followed by decode instructions of both of the thread's chunks
+                // (and one of this step's global loads), the two LDS stores of the decoded
+                // chunks last.  Second slice: fragment reads, one MFMA, the LDS stores of the
+                // states, the remaining MFMAs -- every store of the step then has most of a
+                // slice to complete before the barrier asks for it.
+                if (ks == 0) {
+                    __builtin_amdgcn_sched_group_barrier(0x100, TM + TN + (SPARSE ? 4 : 0), 0);
 #pragma unroll
-                for (int e = 0; e < TM * TN; ++e) {
+                    for (int e = 0; e < TM * TN; ++e) {
+                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                        __builtin_amdgcn_sched_group_barrier(0x002, TM == 4 ? 6 : 12, 0);
+                        if (e < A_LOADS + NWORDS + (SPARSE ? 3 : 2)) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+                    }
+                    __builtin_amdgcn_sched_group_barrier(0x200, 2, 0);
+                } else {
+                    __builtin_amdgcn_sched_group_barrier(0x100, TM + TN, 0);
                     __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                    __builtin_amdgcn_sched_group_barrier(0x002, TM == 4 ? 3 : 6, 0);
-                    if (ks == 0 && e < A_LOADS + NWORDS + (SPARSE ? 3 : 2)) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x200, A_LOADS, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x008, TM * TN - 1, 0);
                 }
-                if (ks == 0) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
-                else __builtin_amdgcn_sched_group_barrier(0x200, 1 + A_LOADS, 0);
             }
             // this step's LDS stores are complete; then all waves meet
             __builtin_amdgcn_s_waitcnt(0xC07F);      // lgkmcnt(0) only
