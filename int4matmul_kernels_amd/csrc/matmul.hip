@@ -403,17 +403,22 @@ __device__ __forceinline__ void pipe_tile(const MatmulArgs& a, const int m0, con
     // (launcher's duty).
     struct AStage { u32x4 v[A_LOADS]; };
     const int a_row = t >> 2, a_chunk = t & 3;
-    // every global address is a workgroup-uniform 64-bit base that moves with the
-    // K step (scalar registers) plus a per-lane 32-bit byte offset that never changes
-    const char* const a_tile = reinterpret_cast<const char*>(x + (int64_t)m0 * a.K);
+    // every global address is a buffer resource (the tile's rows of states; the whole
+    // of the packed matrix, mask, scales, zeros) plus a per-lane 32-bit byte offset that
+    // never changes plus a workgroup-uniform 32-bit offset that moves with the K step:
+    // buffer loads add the three themselves, no address arithmetic is left to the VALU
+    // (the launcher admits only shapes whose tensors stay below 4 GB)
+    constexpr int RSRC_FLAGS = 0x00020000;               // raw buffer, 32-bit data format
+    const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<h16*>(x + (int64_t)m0 * a.K), 0, min(a.M - m0, BM) * a.K * 2, RSRC_FLAGS);
     uint32_t a_off[A_LOADS];
 #pragma unroll
     for (int i = 0; i < A_LOADS; ++i)
         a_off[i] = (uint32_t)((min(a_row + A_ROWS * i, a.M - 1 - m0) * a.K + a_chunk * 8) * 2);
     const int a_dst = a_row * PK + ((a_chunk ^ ((a_row >> 2) & 3)) << 3);       // halves; rows + A_ROWS: same swizzle
-    auto load_a = [&](AStage& r, const char* base) {
+    auto load_a = [&](AStage& r, uint32_t step_off) {
 #pragma unroll
-        for (int i = 0; i < A_LOADS; ++i) r.v[i] = *reinterpret_cast<const u32x4*>(base + a_off[i]);
+        for (int i = 0; i < A_LOADS; ++i) r.v[i] = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, a_off[i], step_off, 0);
     };
     auto write_a = [&](const AStage& r, int stage) {
 #pragma unroll
@@ -440,25 +445,31 @@ __device__ __forceinline__ void pipe_tile(const MatmulArgs& a, const int m0, con
     for (int i = 0; i < NWORDS; ++i)
         b_off[i] = (uint32_t)((((SPARSE ? 0 : BITS == 4 ? 2 * bhb : bhb) + i) * a.S + bcol) * 4);
     const uint32_t m_off = (uint32_t)(bcol * 4);
-    const int64_t m_step = (int64_t)4 * a.S;             // bytes of one row of mask words
+    const uint32_t m_step = 4u * a.S;                    // bytes of one row of mask words
     const uint32_t sz_off = (uint32_t)((bcol & ~1) * 2);
-    const int64_t b_step = (int64_t)(F::ROWS * 4) * a.S;  // bytes of packed weights per K step
-    const int64_t g_step = (int64_t)2 * a.S;             // bytes of one row of scales / zeros
-    // cursor over K steps: packed-weight rows and the scale / zero row of the step's group
-    struct Cursor { const char* w; const char* m; const char* sc; const char* ze; int kt, left; };
+    const uint32_t b_step = (uint32_t)(F::ROWS * 4) * a.S;   // bytes of packed weights per K step
+    const uint32_t g_step = 2u * a.S;                    // bytes of one row of scales / zeros
+    const int k_blocks = a.K / PK, n_groups = (k_blocks + a.group_units * 2 - 1) / (a.group_units * 2);
+    const __amdgpu_buffer_rsrc_t w_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint32_t*>(a.matrix), 0, (int)(k_blocks * b_step), RSRC_FLAGS);
+    const __amdgpu_buffer_rsrc_t m_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint32_t*>(SPARSE ? a.mask : a.matrix), 0, (int)(k_blocks * m_step), RSRC_FLAGS);
+    const __amdgpu_buffer_rsrc_t sc_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<h16*>(a.scales), 0, (int)(n_groups * g_step), RSRC_FLAGS);
+    const __amdgpu_buffer_rsrc_t ze_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<h16*>(a.zeros), 0, (int)(n_groups * g_step), RSRC_FLAGS);
+    // cursor over K steps: byte offsets of the step's packed-weight rows, mask row and scale / zero row
+    struct Cursor { uint32_t w, m, sz; int kt, left; };
     auto cursor_at = [&](int kt) {
         const int gu = a.group_units * 2, group = kt / gu;
-        return Cursor{reinterpret_cast<const char*>(a.matrix) + kt * b_step,
-                      reinterpret_cast<const char*>(a.mask) + (SPARSE ? kt * m_step : 0),
-                      reinterpret_cast<const char*>(a.scales) + group * g_step,
-                      reinterpret_cast<const char*>(a.zeros) + group * g_step, kt, gu - kt % gu};
+        return Cursor{kt * b_step, SPARSE ? kt * m_step : 0u, group * g_step, kt, gu - kt % gu};
     };
     auto load_b = [&](Stage& s, const Cursor& c) {
 #pragma unroll
-        for (int i = 0; i < NWORDS; ++i) s.w[i] = *reinterpret_cast<const uint32_t*>(c.w + b_off[i]);
-        if constexpr (SPARSE) s.m = *reinterpret_cast<const uint32_t*>(c.m + m_off);
-        s.sc = *reinterpret_cast<const uint32_t*>(c.sc + sz_off);
-        s.ze = *reinterpret_cast<const uint32_t*>(c.ze + sz_off);
+        for (int i = 0; i < NWORDS; ++i) s.w[i] = __builtin_amdgcn_raw_buffer_load_b32(w_rsrc, b_off[i], c.w, 0);
+        if constexpr (SPARSE) s.m = __builtin_amdgcn_raw_buffer_load_b32(m_rsrc, m_off, c.m, 0);
+        s.sc = __builtin_amdgcn_raw_buffer_load_b32(sc_rsrc, sz_off, c.sz, 0);
+        s.ze = __builtin_amdgcn_raw_buffer_load_b32(ze_rsrc, sz_off, c.sz, 0);
     };
     auto stage_scale = [&](const Stage& s) { return as_h2(__builtin_amdgcn_perm(s.sc, s.sc, half_sel)); };
     auto stage_negzero = [&](const Stage& s) {
@@ -579,11 +590,10 @@ __device__ __forceinline__ void pipe_tile(const MatmulArgs& a, const int m0, con
             cur.kt += more ? 1 : 0;
             cur.w += more ? b_step : 0;
             if constexpr (SPARSE) cur.m += more ? m_step : 0;
-            cur.sc += wrap ? g_step : 0;
-            cur.ze += wrap ? g_step : 0;
+            cur.sz += wrap ? g_step : 0;
             cur.left = wrap ? a.group_units * 2 : cur.left - (more ? 1 : 0);
         };
-        const char* a_cur = a_tile;
+        uint32_t a_cur = 0;
         int a_kt = 0;
         auto advance_a = [&]() {
             const bool more = a_kt < last;
@@ -666,7 +676,7 @@ __device__ __forceinline__ void pipe_tile(const MatmulArgs& a, const int m0, con
         AStage ra;
         h16x8 fa[TM], fb[TN];
         for (int kt = 0; kt < ktiles; ++kt) {
-            load_a(ra, a_tile + kt * (PK * 2));
+            load_a(ra, (uint32_t)kt * (PK * 2));
             load_b(r, cursor_at(kt));
             write_a(ra, 0);
             write_b_general(r, 0, 0);
@@ -757,8 +767,12 @@ static void launch(const MatmulArgs& a, int64_t B, hipStream_t st) {
     // (M is padded to whole tiles; worth it while the padding stays below an eighth of M,
     // and for a single row of tiles from 161 rows on)
     const int64_t m_pad = (a.M + 255) / 256 * 256;
-    // (the kernel's per-lane byte offsets are 32-bit: 256 rows of states, 4 packed rows of weights)
-    const bool m_ok = ((m_pad - a.M) * 8 <= a.M || (a.M > 160 && a.M <= 256)) && a.K <= (1 << 22) && a.S <= (1 << 27);
+    // (the kernel addresses with 32-bit byte offsets into buffer resources: 256 rows of states,
+    // the whole packed matrix and the whole of scales / zeros have to stay below 2 GB each)
+    const int64_t w_bytes = (int64_t)a.K / 32 * PipeFmt<BITS, SPARSE>::ROWS * 4 * a.S;
+    const int64_t sz_bytes = ((int64_t)a.K / 64 + a.group_units - 1) / a.group_units * a.S * 2;
+    const bool m_ok = ((m_pad - a.M) * 8 <= a.M || (a.M > 160 && a.M <= 256)) && a.K <= (1 << 22) && a.S <= (1 << 27) &&
+                      w_bytes < (1ll << 31) && sz_bytes < (1ll << 31);
     const bool pipe2_ok = !SPARSE && m_ok && a.S % 128 == 0;
     const bool pipe4_ok = m_ok && a.S % 256 == 0;
     if (variant != 1 && variant != 3 && variant != 5 && variant != 6) variant = 0;
