@@ -757,10 +757,10 @@ template <int BITS, bool SPARSE>
 static void launch(const MatmulArgs& a, int64_t B, hipStream_t st) {
     // variant 0 = automatic.  Tile-aligned shapes take the pipelined kernel, as
     // 256 x 256 tiles (one eight-wave workgroup per CU) or 256 x 128 tiles (two
-    // four-wave workgroups per CU).  Measured on MI355X: the large tiles win when
-    // they fill their last round of 256 well; the small ones when fewer than half
-    // of the CUs would get a large tile, or when the large tiles' last round is at
-    // most half full.  The 16:32 format always takes the large tiles (its decode
+    // four-wave workgroups per CU).  Measured on MI355X (K = 4096 ... 20480, S = 5120
+    // ... 28672, M = 256 ... 4096): the small tiles win when at most half of the CUs
+    // would get a large tile, and in the second round of large tiles while it is at
+    // most three eighths full; the large ones everywhere else.  The 16:32 format always takes the large tiles (its decode
     // needs more registers than the four-wave shape leaves).  Everything else:
     // 128 x 256 tiles, and 128 x 128 for narrow outputs or few rows.
     int variant = (int)tuning(TUNE_MM_VARIANT);
