@@ -584,21 +584,24 @@ __device__ __forceinline__ void pipe_tile(const MatmulArgs& a, const int m0, con
         // (selects instead of branches: a branch here would split the scheduling
         // region of the step and invite the compiler to reuse the previous step's
         // scale / zero registers, which makes the step wait for its newest loads)
+        // (plain integer arithmetic on purpose: conditions kept as booleans come out as
+        // 64-bit lane-mask operations, several scalar instructions each)
+        const int gu2 = a.group_units * 2;
         auto advance = [&]() {
-            const bool more = cur.kt < last;
-            const bool wrap = more && cur.left == 1;
-            cur.kt += more ? 1 : 0;
-            cur.w += more ? b_step : 0;
-            if constexpr (SPARSE) cur.m += more ? m_step : 0;
-            cur.sz += wrap ? g_step : 0;
-            cur.left = wrap ? a.group_units * 2 : cur.left - (more ? 1 : 0);
+            const int more = min(last - cur.kt, 1);                  // 1 until the last step is reached
+            const int wrap = cur.left == 1 ? more : 0;
+            cur.kt += more;
+            cur.w += more * b_step;
+            if constexpr (SPARSE) cur.m += more * m_step;
+            cur.sz += wrap * g_step;
+            cur.left += wrap * gu2 - more;
         };
         uint32_t a_cur = 0;
         int a_kt = 0;
         auto advance_a = [&]() {
-            const bool more = a_kt < last;
-            a_kt += more ? 1 : 0;
-            a_cur += more ? PK * 2 : 0;
+            const int more = min(last - a_kt, 1);
+            a_kt += more;
+            a_cur += more * (PK * 2);
         };
         Stage r[3];
         AStage ra[2];
