@@ -384,7 +384,12 @@ template <> struct PipeFmt<4, true> { static constexpr int ROWS = 2, NWORDS = 2;
 
 constexpr int P_STAGES = 3;
 
-template <int BITS, bool SPARSE, int TM, int NW>
+// PING: the waves of the first half ("compute first") run a step as its 16 MFMAs back to back
+// and then everything else; the waves of the second half run everything else first and the MFMAs
+// last.  A SIMD holds one wave of each kind, so its matrix pipe is fed by one wave at a time while
+// the other loads, decodes and stores -- instead of both competing for it and the younger one
+// finishing the step alone.
+template <int BITS, bool SPARSE, int TM, int NW, bool PING>
 __device__ __forceinline__ void pipe_tile(const MatmulArgs& a, const int m0, const int s0, const h16* x,
                                           h16* outs, h16* As, h16* Bs, uint32_t* lut) {
     constexpr int BM = TM * 64, BN = NW * 64, WM = TM * 32, WN = 64, TN = 2, T = 2 * NW * 64;
@@ -652,6 +657,57 @@ __device__ __forceinline__ void pipe_tile(const MatmulArgs& a, const int m0, con
             __builtin_amdgcn_s_waitcnt(0xC07F);      // lgkmcnt(0) only
             __builtin_amdgcn_s_barrier();
         };
+        // the same step in the two orders of PING (phase = 0: MFMAs first; 1: MFMAs last).  Compute-first
+        // waves enter with the step's fragments (both slices) in registers and leave with the next step's;
+        // the others fetch the step's own fragments at its start.
+        auto body_ping = [&](auto phase_tag, int b, AStage& ra_new, const AStage& ra_wr, Stage& r_new, const Stage& r_dec) {
+            constexpr int phase = decltype(phase_tag)::value;
+            const int b1 = (b + 1) % P_STAGES, b2 = (b + 2) % P_STAGES;
+            if constexpr (phase == 0) {
+                mfma_slice(fa[0], fb[0]);
+                mfma_slice(fa[1], fb[1]);
+            }
+            load_frags(phase == 0 ? b1 : b, 0, fa[0], fb[0]);
+            load_frags(phase == 0 ? b1 : b, 1, fa[1], fb[1]);
+            load_a(ra_new, a_cur);             // step kt + 3
+            load_b(r_new, cur);                // step kt + 4
+            advance_a();
+            advance();
+            write_b_fast(r_dec, b2, 0);
+            write_b_fast(r_dec, b2, 1);
+            write_a(ra_wr, b2);
+            if constexpr (phase == 1) {
+                mfma_slice(fa[0], fb[0]);
+                mfma_slice(fa[1], fb[1]);
+            }
+            // scheduling template: the MFMAs as one cluster with the decode instructions in their
+            // shadow (an MFMA occupies the pipe for 32 cycles, the wave issues three or four other
+            // instructions meanwhile); fragment reads, global loads and LDS stores outside it
+            if constexpr (phase == 0) {
+#pragma unroll
+                for (int e = 0; e < 2 * TM * TN; ++e) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);
+                }
+                __builtin_amdgcn_sched_group_barrier(0x100, 2 * (TM + TN) + (SPARSE ? 4 : 0), 0);
+                __builtin_amdgcn_sched_group_barrier(0x020, A_LOADS + NWORDS + (SPARSE ? 3 : 2), 0);
+                __builtin_amdgcn_sched_group_barrier(0x200, A_LOADS + 2, 0);
+            } else {
+                __builtin_amdgcn_sched_group_barrier(0x100, 2 * (TM + TN) + (SPARSE ? 4 : 0), 0);
+                __builtin_amdgcn_sched_group_barrier(0x020, A_LOADS + NWORDS + (SPARSE ? 3 : 2), 0);
+                __builtin_amdgcn_sched_group_barrier(0x200, A_LOADS, 0);
+#pragma unroll
+                for (int e = 0; e < 2 * TM * TN; ++e) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);
+                }
+                __builtin_amdgcn_sched_group_barrier(0x200, 2, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);       // nothing of this step moves behind the barrier
+            __builtin_amdgcn_s_waitcnt(0xC07F);      // lgkmcnt(0) only
+            __builtin_amdgcn_s_barrier();
+            __builtin_amdgcn_sched_barrier(0);
+        };
         load_a(ra[0], a_cur); advance_a();
         load_a(ra[1], a_cur); advance_a();
         load_b(r[0], cur); advance();
@@ -667,11 +723,29 @@ __device__ __forceinline__ void pipe_tile(const MatmulArgs& a, const int m0, con
         load_frags(0, 0, fa[0], fb[0]);
         // LDS stages and weight registers rotate with period 3, state registers with
         // period 2: six steps per trip, unrolled so that all of them are compile-time names
-        for (int kt = 0; kt < ktiles; kt += 6) {
+        if constexpr (!PING) {
+            for (int kt = 0; kt < ktiles; kt += 6) {
 #pragma unroll
-            for (int u = 0; u < 6; ++u) {
-                if (u > 0 && kt + u >= ktiles) break;
-                body(u % 3, ra[(u + 1) % 2], ra[u % 2], r[(u + 1) % 3], r[(u + 2) % 3]);
+                for (int u = 0; u < 6; ++u) {
+                    if (u > 0 && kt + u >= ktiles) break;
+                    body(u % 3, ra[(u + 1) % 2], ra[u % 2], r[(u + 1) % 3], r[(u + 2) % 3]);
+                }
+            }
+        } else {
+            auto run = [&](auto phase_tag) {
+                for (int kt = 0; kt < ktiles; kt += 6) {
+#pragma unroll
+                    for (int u = 0; u < 6; ++u) {
+                        if (u > 0 && kt + u >= ktiles) break;
+                        body_ping(phase_tag, u % 3, ra[(u + 1) % 2], ra[u % 2], r[(u + 1) % 3], r[(u + 2) % 3]);
+                    }
+                }
+            };
+            if (__builtin_amdgcn_readfirstlane(wave) < NW) {
+                load_frags(0, 1, fa[1], fb[1]);
+                run(std::integral_constant<int, 0>{});
+            } else {
+                run(std::integral_constant<int, 1>{});
             }
         }
     } else {
@@ -706,7 +780,7 @@ __device__ __forceinline__ void pipe_tile(const MatmulArgs& a, const int m0, con
         }
 }
 
-template <int BITS, bool SPARSE, int NW, int TM>
+template <int BITS, bool SPARSE, int NW, int TM, bool PING>
 __global__ __launch_bounds__(NW * 128, NW == 2 ? 2 : 1) void matmul_kernel_pipe(MatmulArgs a) {
     constexpr int BM = TM * 64, BN = NW * 64;
     __shared__ __attribute__((aligned(16))) h16 As[P_STAGES * BM * PK];
@@ -735,17 +809,17 @@ __global__ __launch_bounds__(NW * 128, NW == 2 ? 2 : 1) void matmul_kernel_pipe(
         tile_m = bid % a.tiles_m, tile_n = bid / a.tiles_m;
     }
     const int64_t boff = blockIdx.z;
-    pipe_tile<BITS, SPARSE, TM, NW>(a, tile_m * BM, tile_n * BN, a.x + boff * a.M * (int64_t)a.K,
+    pipe_tile<BITS, SPARSE, TM, NW, PING>(a, tile_m * BM, tile_n * BN, a.x + boff * a.M * (int64_t)a.K,
                                    a.outs + boff * a.M * (int64_t)a.S, As, Bs, Lut);
 }
 
-template <int BITS, bool SPARSE, int NW, int TM = 4>
+template <int BITS, bool SPARSE, int NW, int TM = 4, bool PING = false>
 static void launch_pipe(MatmulArgs a, int64_t B, hipStream_t st) {
     a.tiles_m = (a.M + TM * 64 - 1) / (TM * 64);
     a.tiles_n = a.S / (NW * 64);
     const dim3 grid(a.tiles_m * a.tiles_n, 1, (unsigned)B), block(NW * 128);
     a.by_columns = a.tiles_n % 8 == 0;
-    hipLaunchKernelGGL((matmul_kernel_pipe<BITS, SPARSE, NW, TM>), grid, block, 0, st, a);
+    hipLaunchKernelGGL((matmul_kernel_pipe<BITS, SPARSE, NW, TM, PING>), grid, block, 0, st, a);
 }
 
 template <int BITS, bool SPARSE, int BM, int BN, int WM, int WN>
@@ -778,8 +852,8 @@ static void launch(const MatmulArgs& a, int64_t B, hipStream_t st) {
                       w_bytes < (1ll << 31) && sz_bytes < (1ll << 31);
     const bool pipe2_ok = !SPARSE && m_ok && a.S % 128 == 0;
     const bool pipe4_ok = m_ok && a.S % 256 == 0;
-    if (variant != 1 && variant != 3 && variant != 5 && variant != 6) variant = 0;
-    if ((variant == 5 && !pipe2_ok) || (variant == 6 && !pipe4_ok)) variant = 0;
+    if (variant != 1 && variant != 3 && variant != 5 && variant != 6 && variant != 9) variant = 0;
+    if ((variant == 5 && !pipe2_ok) || ((variant == 6 || variant == 9) && !pipe4_ok)) variant = 0;
     if (variant == 0) {
         const int64_t tiles4 = m_pad / 256 * (a.S / 256) * B;
         const int64_t last = tiles4 % 256;
@@ -791,7 +865,10 @@ static void launch(const MatmulArgs& a, int64_t B, hipStream_t st) {
     }
     if (variant == 1) launch_tile<BITS, SPARSE, 128, 128, 64, 64>(a, B, st);
     else if (variant == 3) launch_tile<BITS, SPARSE, 128, 256, 128, 64>(a, B, st);
-    else if (variant == 6) launch_pipe<BITS, SPARSE, 4>(a, B, st);
+    // (256 x 256: the dense formats run the two halves of the workgroup in opposite phases, 2-3 %
+    // faster; the 16:32 decode has no registers to spare for it.  Variant 9 forces the plain order.)
+    else if (variant == 6 && !SPARSE) launch_pipe<BITS, SPARSE, 4, 4, true>(a, B, st);
+    else if (variant == 6 || variant == 9) launch_pipe<BITS, SPARSE, 4>(a, B, st);
     else if constexpr (!SPARSE) launch_pipe<BITS, false, 2>(a, B, st);
 }
 

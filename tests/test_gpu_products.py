@@ -189,13 +189,17 @@ def test_full_size_matvec_and_matmul_c2_c3(H):
 
 
 @pytest.mark.parametrize("bits,sparse,variant", [(4, False, 5), (3, False, 5), (2, False, 5), (4, False, 6),
-                                                 (3, False, 6), (2, False, 6), (4, True, 6)])
-@pytest.mark.parametrize("M,K,S,g,B", [(256, 512, 512, 128, 1), (512, 192, 256, 64, 2), (256, 2048, 256, -1, 1)])
+                                                 (3, False, 6), (2, False, 6), (4, True, 6), (4, False, 9),
+                                                 (3, False, 9), (2, False, 9)])
+@pytest.mark.parametrize("M,K,S,g,B", [(256, 512, 512, 128, 1), (512, 192, 256, 64, 2), (256, 2048, 256, -1, 1),
+                                       (512, 448, 512, 64, 1)])
 def test_pipelined_matmul_with_exponent_groups(H, bits, sparse, variant, M, K, S, g, B):
     """tile-aligned dense shapes take the pipelined kernel (variant 5: 256 x 128
-    tiles, variant 6: 256 x 256); negative scales in a few columns force its
-    general loop for the tiles that contain them.  K = 192 is six K steps (one
-    trip of the unrolled loop), K = 2048 with a single group runs many trips."""
+    tiles, variant 6: 256 x 256 with the two halves of the workgroup in opposite
+    phases for the dense formats, variant 9: 256 x 256 in the plain order); negative
+    scales in a few columns force its general loop for the tiles that contain them.
+    K = 192 is six K steps (one trip of the unrolled loop), K = 448 fourteen (two trips
+    and a remainder), K = 2048 with a single group runs many trips."""
     from int4matmul_kernels_amd import capi
     p = O.make_problem(K=K, S=S, M=M, bits=bits, group_size=g, sparse=sparse, seed=21 + bits, B=B)
     capi.tune(3, variant)
