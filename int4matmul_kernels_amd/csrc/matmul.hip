@@ -857,7 +857,7 @@ static void launch(const MatmulArgs& a, int64_t B, hipStream_t st) {
     if (variant == 0) {
         const int64_t tiles4 = m_pad / 256 * (a.S / 256) * B;
         const int64_t last = tiles4 % 256;
-        const bool small_better = tiles4 < 128 || (tiles4 > 256 && last > 0 && last <= 128);
+        const bool small_better = tiles4 <= 128 || (tiles4 > 256 && tiles4 < 512 && last > 0 && last <= 96);
         if (pipe4_ok && (SPARSE || !pipe2_ok || !small_better)) variant = 6;
         else if (pipe2_ok) variant = 5;
         else if (a.M > 512 && a.S >= 256) variant = 3;
