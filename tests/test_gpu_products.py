@@ -90,7 +90,8 @@ def test_degenerate_known_answer(H, bits, sparse, K):
 # ------------------------------------------------------------------- matmul
 @pytest.mark.parametrize("bits,sparse", FORMATS)
 @pytest.mark.parametrize("M,K,S,g", [(2048, 128, 128, 128), (70, 256, 192, 64), (1, 512, 64, 128), (500, 192, 256, 64),
-                                     (257, 1024, 320, -1)])
+                                     (257, 1024, 320, -1), (342, 256, 512, 64), (400, 320, 256, 64), (600, 128, 384, 128),
+                                     (700, 192, 256, 64)])
 def test_matmul_parity(H, bits, sparse, M, K, S, g):
     p = _problem(bits, sparse, K=K, S=S, M=M, group_size=g, seed=M)
     d = H.dev_problem(p)
