@@ -30,6 +30,8 @@ MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 MFMA
 # HBM bytes per matvec launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see
 # profiles/matvec_int4_K5120_S20480.md)
 MATVEC_TRAFFIC_BYTES = 57_508_864  # (27580.5 KiB x 2.000 + 1000.0 KiB x 1.000) x 1024
+# the same for the M=2048 matmul (profiles/matmul_int4_M2048_K5120_S20480.md)
+MATMUL_TRAFFIC_BYTES = 465_845_248  # (185900.4 KiB x 2.000 + 83127.1 KiB x 1.000) x 1024
 
 
 def matvec_bytes(K, S, g, bits=4):
@@ -188,7 +190,7 @@ def main():
                           "us": round(mm_us, 2), "tflops": round(tf, 1),
                           "roofline": {"bound": "mfma", "achieved": round(tf, 1), "peak": MFMA_FP16_PEAK_TFLOPS,
                                        "unit": "TFLOP/s", "frac": round(tf / MFMA_FP16_PEAK_TFLOPS, 4),
-                                       "traffic": None},
+                                       "traffic": MATMUL_TRAFFIC_BYTES},
                           "max_rel_err_vs_fp32_oracle": float(f"{mm_err:.3e}")}
 
     # ---- CPU baseline: torch dequantise + fp32 matmul on the host (reported only)
