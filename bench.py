@@ -31,7 +31,7 @@ MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 MFMA
 # profiles/matvec_int4_K5120_S20480.md)
 MATVEC_TRAFFIC_BYTES = 57_508_864  # (27580.5 KiB x 2.000 + 1000.0 KiB x 1.000) x 1024
 # the same for the M=2048 matmul (profiles/matmul_int4_M2048_K5120_S20480.md)
-MATMUL_TRAFFIC_BYTES = 465_845_248  # (185900.4 KiB x 2.000 + 83127.1 KiB x 1.000) x 1024
+MATMUL_TRAFFIC_BYTES = 465_846_170  # (185900.4 KiB x 2.000 + 83127.1 KiB x 1.000) x 1024
 
 
 def matvec_bytes(K, S, g, bits=4):
