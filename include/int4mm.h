@@ -71,7 +71,8 @@ INT4MM_API int int4mm_abi_version(void);
  * group, 2 = matvec lane groups per wave (1, 2, 4), 3 = matmul kernel variant
  * (5 / 6 = pipelined 256x128 / 256x256 tiles, 9 = 256x256 without the two-phase
  * order), 4 = matvec: 1 disables prefetch,
- * 5 = 1 disables the few-row (2..96 rows) kernel. */
+ * 5 = 1 disables the few-row (2..96 rows) kernel, 6 = matmul split-K factor
+ * (1 = never split, 2..8 = that factor where the shape allows a split at all). */
 INT4MM_API int int4mm_tune(int key, int64_t value);
 
 /* Shape of one product.  matrix_rows = R, n_groups = G (rows of scales/zeros).
@@ -98,6 +99,14 @@ typedef struct int4mm_shape {
  * Calls that share one workspace must not overlap in time. */
 INT4MM_API size_t int4mm_workspace_bytes(int64_t max_out_size);
 INT4MM_API int int4mm_workspace_init(void* workspace, size_t workspace_bytes, void* stream);
+
+/* Bytes of workspace with which int4mm_matmul may split the K dimension of `shape`
+ * over several workgroups per output tile (shapes with so few tiles that most of
+ * the GPU would idle; `sparse` != 0 for the 16:32 format); never less than
+ * int4mm_workspace_bytes(shape->out_size).  A smaller workspace is not an error:
+ * the product then runs unsplit.  Same zero-fill rule as above.  No counterpart in
+ * the reference, whose matmul (matmul_kernel.cu:375-459) uses no scratch. */
+INT4MM_API size_t int4mm_matmul_workspace_bytes(const int4mm_shape* shape, int sparse);
 
 /* Matrix-vector product, M == 1 per batch entry:
  *     outs[b,0,:] = fp16( fp32(outs[b,0,:]) + multiplier[b,0,:] @ W )

@@ -14,7 +14,7 @@ LIB_NAME = "libint4mm_hip.so"
 
 EXPORTS = [
     "int4mm_error_string", "int4mm_last_hip_error", "int4mm_abi_version", "int4mm_tune",
-    "int4mm_workspace_bytes", "int4mm_workspace_init", "int4mm_matvec", "int4mm_matmul",
+    "int4mm_workspace_bytes", "int4mm_workspace_init", "int4mm_matmul_workspace_bytes", "int4mm_matvec", "int4mm_matmul",
     "int4mm_sparse_pack", "int4mm_dense_pack", "int4mm_unpack", "int4mm_dequantize",
 ]
 
@@ -53,6 +53,8 @@ def lib():
     L.int4mm_tune.argtypes = [C.c_int, i64]
     L.int4mm_workspace_bytes.restype = sz
     L.int4mm_workspace_bytes.argtypes = [i64]
+    L.int4mm_matmul_workspace_bytes.restype = sz
+    L.int4mm_matmul_workspace_bytes.argtypes = [C.POINTER(Shape), C.c_int]
     L.int4mm_workspace_init.restype = C.c_int
     L.int4mm_workspace_init.argtypes = [vp, sz, vp]
     for name in ("int4mm_matvec", "int4mm_matmul"):
@@ -93,6 +95,17 @@ def new_workspace(out_size: int, device="cuda"):
     import torch
     n = lib().int4mm_workspace_bytes(out_size)
     return torch.zeros(n, dtype=torch.uint8, device=device)
+
+
+def matmul_workspace_bytes(batch, seq_len, in_size, out_size, sparse=False) -> int:
+    """bytes of workspace with which `matmul` may split K for this shape"""
+    sh = Shape(batch, seq_len, in_size, out_size, 0, 0, 0)
+    return lib().int4mm_matmul_workspace_bytes(C.byref(sh), 1 if sparse else 0)
+
+
+def new_matmul_workspace(batch, seq_len, in_size, out_size, sparse=False, device="cuda"):
+    import torch
+    return torch.zeros(matmul_workspace_bytes(batch, seq_len, in_size, out_size, sparse), dtype=torch.uint8, device=device)
 
 
 def _shape(outs, matrix, multiplier, scales, group_size):

@@ -54,8 +54,9 @@ struct Scratch { torch::Tensor buf; };
 std::mutex g_mu;
 std::map<std::pair<int, int64_t>, Scratch> g_scratch;
 
-torch::Tensor workspace_for(const c10::Device& dev, c10::hip::HIPStream stream, int64_t out_size) {
-    const size_t need = int4mm_workspace_bytes(out_size);
+torch::Tensor workspace_for(const c10::Device& dev, c10::hip::HIPStream stream, const int4mm_shape& shape, bool sparse) {
+    // (covers the matvec's need; more when a matmul of this shape wants to split K)
+    const size_t need = int4mm_matmul_workspace_bytes(&shape, sparse ? 1 : 0);
     std::lock_guard<std::mutex> lock(g_mu);
     auto key = std::make_pair((int)dev.index(), (int64_t)stream.id());
     auto it = g_scratch.find(key);
@@ -119,7 +120,7 @@ Prepared prepare(TENSOR_MULT_ARGS, torch::Tensor& ws_keepalive) {
     p.mask = is_sparse ? sparse_mask.value().data_ptr() : nullptr;
     auto stream = c10::hip::getCurrentHIPStream(dev.index());
     p.stream = stream.stream();
-    ws_keepalive = workspace_for(dev, stream, S);
+    ws_keepalive = workspace_for(dev, stream, p.shape, is_sparse);
     p.ws = ws_keepalive.data_ptr();
     p.ws_bytes = (size_t)ws_keepalive.numel();
     return p;

@@ -22,6 +22,7 @@
 // disjoint column ranges of the weight matrix.
 #include "common.h"
 
+#include <algorithm>
 #include <type_traits>
 
 namespace i4 {
@@ -42,6 +43,12 @@ struct MatmulArgs {
     int group_units;        // group size / 64
     int tiles_m, tiles_n;
     int by_columns;         // pipelined kernel: 1 = an XCD walks its range of tile columns row by row
+    // split-K (pipelined kernel, grids that would leave most of the GPU idle): `ksplit` workgroups
+    // share a tile, each walks 1 / ksplit of the K steps and stores its fp32 partial tile to
+    // `part`; the one that arrives last (`counters`, one per tile) adds them up in split order
+    int ksplit;
+    float* part;
+    int* counters;
 };
 
 // Raw packed data of one (32-row block, column) cell
@@ -389,9 +396,9 @@ constexpr int P_STAGES = 3;
 // last.  A SIMD holds one wave of each kind, so its matrix pipe is fed by one wave at a time while
 // the other loads, decodes and stores -- instead of both competing for it and the younger one
 // finishing the step alone.
-template <int BITS, bool SPARSE, int TM, int NW, bool PING>
+template <int BITS, bool SPARSE, int TM, int NW, bool PING, bool SPLIT>
 __device__ __forceinline__ void pipe_tile(const MatmulArgs& a, const int m0, const int s0, const h16* x,
-                                          h16* outs, h16* As, h16* Bs, uint32_t* lut) {
+                                          h16* outs, h16* As, h16* Bs, uint32_t* lut, const int tile, const int split) {
     constexpr int BM = TM * 64, BN = NW * 64, WM = TM * 32, WN = 64, TN = 2, T = 2 * NW * 64;
     constexpr int A_STAGE = BM * PK, B_STAGE = PK * BN;            // halves per stage
     constexpr int A_ROWS = T / 4;                                  // rows covered by one 16-byte load per thread
@@ -553,8 +560,12 @@ __device__ __forceinline__ void pipe_tile(const MatmulArgs& a, const int m0, con
                 acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[i], fb[j], acc[i][j], 0, 0, 0);
     };
 
-    const int ktiles = a.K / PK;
-    const int last = ktiles - 1;
+    // K steps kt0 .. last of the matrix belong to this workgroup (all of them unless SPLIT)
+    const int ksteps = a.K / PK;
+    const int per_split = SPLIT ? (ksteps + a.ksplit - 1) / a.ksplit : ksteps;
+    const int kt0 = SPLIT ? split * per_split : 0;
+    const int ktiles = SPLIT ? min(ksteps, kt0 + per_split) - kt0 : ksteps;
+    const int last = kt0 + ktiles - 1;
 
     // Does any (group, column) of this tile use exponent quantisation (scale < 0
     // or NaN)?  One pass over the tile's scales (a few KB); the answer is
@@ -574,7 +585,7 @@ __device__ __forceinline__ void pipe_tile(const MatmulArgs& a, const int m0, con
     __syncthreads();
     {
         bool bad = false;
-        const int groups = (ktiles + a.group_units * 2 - 1) / (a.group_units * 2);
+        const int groups = (ksteps + a.group_units * 2 - 1) / (a.group_units * 2);
         for (int g = bhb; g < groups; g += 2) bad |= !(a.scales[(int64_t)g * a.S + bcol] >= (h16)0.0f);
         if (__builtin_amdgcn_ballot_w64(bad) != 0 && lane == 0) any_expo = 1;
     }
@@ -585,7 +596,7 @@ __device__ __forceinline__ void pipe_tile(const MatmulArgs& a, const int m0, con
     if (!tile_has_expo) {
         // Cursors of the loads: weights run four K steps ahead of the MFMAs, states
         // three; both stop at the last step (the surplus loads re-read it, unused).
-        Cursor cur = cursor_at(0);
+        Cursor cur = cursor_at(kt0);
         // (selects instead of branches: a branch here would split the scheduling
         // region of the step and invite the compiler to reuse the previous step's
         // scale / zero registers, which makes the step wait for its newest loads)
@@ -601,8 +612,8 @@ __device__ __forceinline__ void pipe_tile(const MatmulArgs& a, const int m0, con
             cur.sz += wrap * g_step;
             cur.left += wrap * gu2 - more;
         };
-        uint32_t a_cur = 0;
-        int a_kt = 0;
+        uint32_t a_cur = (uint32_t)kt0 * (PK * 2);
+        int a_kt = kt0;
         auto advance_a = [&]() {
             const int more = min(last - a_kt, 1);
             a_kt += more;
@@ -753,8 +764,8 @@ __device__ __forceinline__ void pipe_tile(const MatmulArgs& a, const int m0, con
         AStage ra;
         h16x8 fa[TM], fb[TN];
         for (int kt = 0; kt < ktiles; ++kt) {
-            load_a(ra, (uint32_t)kt * (PK * 2));
-            load_b(r, cursor_at(kt));
+            load_a(ra, (uint32_t)(kt0 + kt) * (PK * 2));
+            load_b(r, cursor_at(kt0 + kt));
             write_a(ra, 0);
             write_b_general(r, 0, 0);
             write_b_general(r, 0, 1);
@@ -766,6 +777,57 @@ __device__ __forceinline__ void pipe_tile(const MatmulArgs& a, const int m0, con
             }
             __syncthreads();
         }
+    }
+    if constexpr (SPLIT) {
+        // Every workgroup of the tile stores its partial accumulators (16 bytes per lane and
+        // store: register group g of thread t at (g * T + t) * 16 -- whole cache lines per wave)
+        // and then counts itself in; whoever finds all the others counted adds the partials up
+        // in split order (its own included, from memory: the sum has one order whoever is
+        // last) and writes the tile.  Stores and loads go straight through to memory
+        // (system-scope cache policy), the counter is a device-scope atomic: no cache-wide
+        // fence, no waiting.
+        constexpr int GROUPS = TM * TN * 4, SLOT_BYTES = BM * BN * 4, THROUGH = 17;      // sc0 | sc1
+        char* const slots = reinterpret_cast<char*>(a.part) + (int64_t)tile * a.ksplit * SLOT_BYTES;
+        const __amdgpu_buffer_rsrc_t mine = __builtin_amdgcn_make_buffer_rsrc(
+            slots + (int64_t)split * SLOT_BYTES, 0, SLOT_BYTES, RSRC_FLAGS);
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const f32x4 v = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+                    __builtin_amdgcn_raw_buffer_store_b128(bitcast<u32x4>(v), mine, (((i * TN + j) * 4 + q) * T + t) * 16, 0, THROUGH);
+                }
+        __builtin_amdgcn_s_waitcnt(0);                 // every store of this thread has been acknowledged
+        int* const flag = reinterpret_cast<int*>(As);
+        __syncthreads();
+        if (t == 0) *flag = __hip_atomic_fetch_add(a.counters + tile, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        if (*flag != a.ksplit - 1) return;
+        if (t == 0) __hip_atomic_store(a.counters + tile, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // clean for the next call
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+        for (int sp = 0; sp < a.ksplit; ++sp) {
+            const __amdgpu_buffer_rsrc_t theirs = __builtin_amdgcn_make_buffer_rsrc(
+                slots + (int64_t)sp * SLOT_BYTES, 0, SLOT_BYTES, RSRC_FLAGS);
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const f32x4 v = bitcast<f32x4>(__builtin_amdgcn_raw_buffer_load_b128(
+                            theirs, (((i * TN + j) * 4 + q) * T + t) * 16, 0, THROUGH));
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) acc[i][j][4 * q + e] += v[e];
+                    }
+        }
+        (void)GROUPS;
     }
 #pragma unroll
     for (int i = 0; i < TM; ++i)
@@ -780,13 +842,15 @@ __device__ __forceinline__ void pipe_tile(const MatmulArgs& a, const int m0, con
         }
 }
 
-template <int BITS, bool SPARSE, int NW, int TM, bool PING>
+template <int BITS, bool SPARSE, int NW, int TM, bool PING, bool SPLIT>
 __global__ __launch_bounds__(NW * 128, NW == 2 ? 2 : 1) void matmul_kernel_pipe(MatmulArgs a) {
     constexpr int BM = TM * 64, BN = NW * 64;
     __shared__ __attribute__((aligned(16))) h16 As[P_STAGES * BM * PK];
     __shared__ __attribute__((aligned(16))) h16 Bs[P_STAGES * PK * BN];
     __shared__ __attribute__((aligned(16))) uint32_t Lut[SPARSE ? SPARSE_LUT_WORDS : 4];
-    int bid = blockIdx.x;
+    // (split-K: the workgroups of a tile are neighbours in the grid, so they run at about the same time)
+    const int split = SPLIT ? (int)blockIdx.x % a.ksplit : 0;
+    int bid = SPLIT ? (int)blockIdx.x / a.ksplit : (int)blockIdx.x;
     const int total = a.tiles_m * a.tiles_n;
     int tile_m, tile_n;
     if (total % 8 == 0) {
@@ -809,17 +873,51 @@ __global__ __launch_bounds__(NW * 128, NW == 2 ? 2 : 1) void matmul_kernel_pipe(
         tile_m = bid % a.tiles_m, tile_n = bid / a.tiles_m;
     }
     const int64_t boff = blockIdx.z;
-    pipe_tile<BITS, SPARSE, TM, NW, PING>(a, tile_m * BM, tile_n * BN, a.x + boff * a.M * (int64_t)a.K,
-                                   a.outs + boff * a.M * (int64_t)a.S, As, Bs, Lut);
+    pipe_tile<BITS, SPARSE, TM, NW, PING, SPLIT>(a, tile_m * BM, tile_n * BN, a.x + boff * a.M * (int64_t)a.K,
+                                          a.outs + boff * a.M * (int64_t)a.S, As, Bs, Lut,
+                                          ((int)boff * a.tiles_n + tile_n) * a.tiles_m + tile_m, split);
 }
 
 template <int BITS, bool SPARSE, int NW, int TM = 4, bool PING = false>
 static void launch_pipe(MatmulArgs a, int64_t B, hipStream_t st) {
     a.tiles_m = (a.M + TM * 64 - 1) / (TM * 64);
     a.tiles_n = a.S / (NW * 64);
-    const dim3 grid(a.tiles_m * a.tiles_n, 1, (unsigned)B), block(NW * 128);
+    const dim3 grid(a.tiles_m * a.tiles_n * a.ksplit, 1, (unsigned)B), block(NW * 128);
     a.by_columns = a.tiles_n % 8 == 0;
-    hipLaunchKernelGGL((matmul_kernel_pipe<BITS, SPARSE, NW, TM, PING>), grid, block, 0, st, a);
+    if constexpr (!PING) {
+        if (a.ksplit > 1) {
+            hipLaunchKernelGGL((matmul_kernel_pipe<BITS, SPARSE, NW, TM, false, true>), grid, block, 0, st, a);
+            return;
+        }
+    }
+    hipLaunchKernelGGL((matmul_kernel_pipe<BITS, SPARSE, NW, TM, PING, false>), grid, block, 0, st, a);
+}
+
+// ---- split-K plan.  Shapes with at most 128 tiles of 256 x 256 leave more than half of the GPU
+// idle; they run as 256 x 128 tiles (16:32: 256 x 256) with `ksplit` workgroups per tile.  The factor
+// minimises a cost in K steps fitted to measurements (K = 4096 ... 20480, 32 ... 240 tiles):
+// rounds of 256 workgroups x (steps per workgroup + 20 for its prologue and hand-over) + 6 per split.
+constexpr int64_t MM_SPLIT_MAX_TILES = 1024;             // counters: one int per tile in 4 KB
+constexpr int64_t MM_SPLIT_MAX_BYTES = 192ll << 20;      // cap of the partial tiles
+struct SplitPlan { int ksplit; int64_t tiles; int64_t tile_bytes; };
+static SplitPlan plan_split(bool sparse, int64_t B, int64_t M, int64_t K, int64_t S) {
+    const SplitPlan none{1, 0, 0};
+    if (S % 256 != 0) return none;
+    const int64_t m_pad = (M + 255) / 256 * 256, tiles4 = m_pad / 256 * (S / 256) * B;
+    if (tiles4 > 128) return none;
+    SplitPlan p{1, sparse ? tiles4 : 2 * tiles4, sparse ? 256 * 256 * 4 : 256 * 128 * 4};
+    if (p.tiles > MM_SPLIT_MAX_TILES) return none;
+    const int64_t steps = K / 32, forced = tuning(TUNE_MM_SPLIT);
+    auto cost = [&](int64_t ks) { return (p.tiles * ks + 255) / 256 * ((steps + ks - 1) / ks + 20) + (ks > 1 ? 6 * ks : 0); };
+    int64_t best = 1;
+    for (int64_t ks = 2; ks <= 8; ++ks) {
+        if (steps / ks < 8 || p.tiles * ks * p.tile_bytes > MM_SPLIT_MAX_BYTES) break;
+        if (forced == ks) { best = ks; break; }
+        if (forced == 0 && cost(ks) < cost(best)) best = ks;
+    }
+    if (best < 2) return none;
+    p.ksplit = (int)best;
+    return p;
 }
 
 template <int BITS, bool SPARSE, int BM, int BN, int WM, int WN>
@@ -831,7 +929,7 @@ static void launch_tile(MatmulArgs a, int64_t B, hipStream_t st) {
 }
 
 template <int BITS, bool SPARSE>
-static void launch(const MatmulArgs& a, int64_t B, hipStream_t st) {
+static void launch(MatmulArgs a, int64_t B, hipStream_t st, void* workspace, size_t workspace_bytes) {
     // variant 0 = automatic.  Tile-aligned shapes take the pipelined kernel, as
     // 256 x 256 tiles (one eight-wave workgroup per CU) or 256 x 128 tiles (two
     // four-wave workgroups per CU).  Measured on MI355X (K = 4096 ... 20480, S = 5120
@@ -864,6 +962,18 @@ static void launch(const MatmulArgs& a, int64_t B, hipStream_t st) {
         else if (a.M > 512 && a.S >= 256) variant = 3;
         else variant = 1;
     }
+    // split-K where the plan asks for it and the caller's workspace has room (it then holds, behind
+    // the matvec's part, one page of per-tile counters and the partial tiles)
+    if ((SPARSE && (variant == 6 || variant == 9)) || (!SPARSE && variant == 5)) {
+        const SplitPlan sp = plan_split(SPARSE, B, a.M, a.K, a.S);
+        const size_t base = int4mm_workspace_bytes(a.S);
+        if (sp.ksplit > 1 && workspace != nullptr &&
+            workspace_bytes >= base + 4096 + (size_t)(sp.tiles * sp.ksplit * sp.tile_bytes)) {
+            a.ksplit = sp.ksplit;
+            a.counters = reinterpret_cast<int*>(static_cast<char*>(workspace) + base);
+            a.part = reinterpret_cast<float*>(static_cast<char*>(workspace) + base + 4096);
+        }
+    }
     if (variant == 1) launch_tile<BITS, SPARSE, 128, 128, 64, 64>(a, B, st);
     else if (variant == 3) launch_tile<BITS, SPARSE, 128, 256, 128, 64>(a, B, st);
     // (256 x 256: the dense formats run the two halves of the workgroup in opposite phases, 2-3 %
@@ -881,7 +991,6 @@ extern "C" int int4mm_matmul(int bits, void* outs, const void* matrix, const voi
                              const void* scales, const void* zeros, const void* sparse_mask,
                              const int4mm_shape* shape, void* workspace, size_t workspace_bytes,
                              void* stream) {
-    (void)workspace; (void)workspace_bytes;
     int rc = validate_product(bits, outs, matrix, multiplier, scales, zeros, sparse_mask, shape, false);
     if (rc != INT4MM_OK) return rc;
     const int64_t B = shape->batch, M = shape->seq_len, K = shape->in_size, S = shape->out_size;
@@ -909,10 +1018,25 @@ extern "C" int int4mm_matmul(int bits, void* outs, const void* matrix, const voi
     a.group_units = (int)(g / 64 > 0x7FFFFFF ? 0x7FFFFFF : g / 64);
     a.tiles_m = a.tiles_n = 0;
     a.by_columns = 0;
+    a.ksplit = 1;
+    a.part = nullptr;
+    a.counters = nullptr;
 
-    if (sparse_mask) launch<4, true>(a, B, st);
-    else if (bits == 4) launch<4, false>(a, B, st);
-    else if (bits == 3) launch<3, false>(a, B, st);
-    else launch<2, false>(a, B, st);
+    if (sparse_mask) launch<4, true>(a, B, st, workspace, workspace_bytes);
+    else if (bits == 4) launch<4, false>(a, B, st, workspace, workspace_bytes);
+    else if (bits == 3) launch<3, false>(a, B, st, workspace, workspace_bytes);
+    else launch<2, false>(a, B, st, workspace, workspace_bytes);
     return check_launch("matmul");
+}
+
+// Workspace with which int4mm_matmul may split K for this shape: the matvec's part, one page of
+// counters and the partial tiles.  A smaller workspace is not an error: the product then runs unsplit.
+extern "C" size_t int4mm_matmul_workspace_bytes(const int4mm_shape* shape, int sparse) {
+    if (shape == nullptr) return 0;
+    const int64_t B = shape->batch, M = shape->seq_len, K = shape->in_size, S = shape->out_size;
+    size_t need = int4mm_workspace_bytes(S);
+    if (B <= 0 || M <= 0 || K < 64 || S < 128) return need;
+    const SplitPlan sp = plan_split(sparse != 0, B, M, K, S);
+    if (sp.ksplit > 1) need += 4096 + (size_t)(sp.tiles * sp.ksplit * sp.tile_bytes);
+    return need;
 }

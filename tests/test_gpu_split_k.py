@@ -1,0 +1,100 @@
+"""Split-K of the pipelined matmul: shapes with few output tiles run several
+workgroups per tile, each over a part of K, and the last one to finish adds the
+fp32 partial tiles up.  Checked against the oracle, against the unsplit kernel
+(tuning key 6 = 1), on repeated calls through one workspace (the per-tile
+counters must come back to zero), with too small a workspace (falls back to the
+unsplit kernel) and through the extension, which sizes its own workspace."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+from oracle import oracle as O  # noqa: E402
+
+
+@pytest.fixture(scope="module")
+def H():
+    from tests import helpers
+    return helpers
+
+
+def _problem(bits, sparse, **kw):
+    if bits != 4:
+        kw.setdefault("scale_range", (0.004, 0.08))
+        kw.setdefault("zero_const", 3.5 if bits == 3 else 1.5)
+    return O.make_problem(bits=bits, sparse=sparse, **kw)
+
+
+FORMATS = [(4, False), (3, False), (2, False), (4, True)]
+
+
+@pytest.mark.parametrize("bits,sparse", FORMATS)
+@pytest.mark.parametrize("M,K,S,g,B", [(256, 2048, 512, 128, 1), (200, 1536, 256, 64, 1), (512, 4096, 256, -1, 1),
+                                       (256, 1024, 256, 64, 3), (400, 2560, 768, 128, 1)])
+def test_split_k_matches_oracle_and_unsplit(H, bits, sparse, M, K, S, g, B):
+    capi = H.capi
+    p = _problem(bits, sparse, K=K, S=S, M=M, group_size=g, seed=M + K, B=B)
+    assert capi.matmul_workspace_bytes(B, M, K, S, sparse) > capi.lib().int4mm_workspace_bytes(S), "shape should split"
+    d = H.dev_problem(p)
+    exact, f32 = H.oracles(p)
+    got = H.run_capi(p, d, "mtx")
+    H.assert_product_close(got, exact, f32, kind="mtx")
+    capi.tune(6, 1)
+    try:
+        ref = H.run_capi(p, d, "mtx")
+    finally:
+        capi.tune(6, 0)
+    assert O.max_rel_error(ref.astype(np.float64), got) < H.TOL_EXACT
+
+
+@pytest.mark.parametrize("bits,sparse", [(4, False), (4, True)])
+def test_split_k_repeated_calls_share_a_workspace(H, bits, sparse):
+    capi = H.capi
+    p = _problem(bits, sparse, K=2048, S=512, M=256, group_size=128, seed=5)
+    d = H.dev_problem(p)
+    ws = capi.new_matmul_workspace(1, 256, 2048, 512, sparse)
+    outs = torch.zeros((1, 256, 512), dtype=torch.float16, device="cuda")
+    results = []
+    for _ in range(4):
+        outs.fill_(7.0)
+        capi.matmul(bits, outs, d["matrix"], d["states"], d["scales"], d["zeros"], 128, d["mask"], ws)
+        torch.cuda.synchronize()
+        results.append(outs.cpu().numpy().copy())
+    for r in results[1:]:
+        assert np.array_equal(r, results[0])              # the sum has one order whoever arrives last
+    exact, f32 = H.oracles(p)
+    H.assert_product_close(results[0], exact, f32, kind="mtx")
+    base = capi.lib().int4mm_workspace_bytes(512)
+    assert int(ws[base:base + 4096].to(torch.int32).sum()) == 0    # the counters are back to zero
+
+
+def test_split_k_needs_room_in_the_workspace(H):
+    capi = H.capi
+    p = _problem(4, False, K=2048, S=512, M=256, group_size=128, seed=6)
+    d = H.dev_problem(p)
+    exact, f32 = H.oracles(p)
+    for ws in (None, capi.new_workspace(512)):            # no room for partial tiles: the unsplit kernel runs
+        outs = torch.zeros((1, 256, 512), dtype=torch.float16, device="cuda")
+        capi.matmul(4, outs, d["matrix"], d["states"], d["scales"], d["zeros"], 128, None, ws)
+        torch.cuda.synchronize()
+        H.assert_product_close(outs.cpu().numpy(), exact, f32, kind="mtx")
+
+
+@pytest.mark.parametrize("bits,sparse", [(4, False), (4, True)])
+def test_split_k_exponent_mode_columns(H, bits, sparse):
+    p = _problem(bits, sparse, K=2048, S=512, M=256, group_size=128, seed=8)
+    p["scales"][3, 40:48] *= np.float16(-1)
+    p["scales"][9, 300] *= np.float16(-1)
+    d = H.dev_problem(p)
+    exact, f32 = H.oracles(p)
+    H.assert_product_close(H.run_capi(p, d, "mtx"), exact, f32, kind="mtx")
+
+
+@pytest.mark.parametrize("bits,sparse", [(4, False), (3, False), (4, True)])
+def test_split_k_through_the_extension(H, bits, sparse):
+    p = _problem(bits, sparse, K=2048, S=512, M=256, group_size=128, seed=9)
+    d = H.dev_problem(p)
+    exact, f32 = H.oracles(p)
+    for _ in range(2):
+        H.assert_product_close(H.run_ext(p, d), exact, f32, kind="mtx")
