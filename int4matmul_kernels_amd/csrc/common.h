@@ -94,6 +94,8 @@ enum TuneKey { TUNE_MV_WAVES = 0, TUNE_MV_UNITS = 1, TUNE_MV_LK = 2, TUNE_MM_VAR
 // few-row product (2 .. 96 rows; sparse_mask != nullptr: 16:32 int4); false = shape not taken, use the general kernels
 bool skinny_rows(int bits, _Float16* outs, const uint32_t* matrix, const _Float16* x, const _Float16* scales,
                  const _Float16* zeros, int64_t R, int64_t K, int64_t S, int64_t group_size, bool accumulate,
-                 hipStream_t st, const uint32_t* sparse_mask);
+                 hipStream_t st, const uint32_t* sparse_mask, void* workspace, size_t workspace_bytes);
+// room the few-row kernel wants behind the matvec's part of the workspace to split K across workgroups (0: none)
+size_t skinny_workspace_bytes(int64_t R, int64_t K, int64_t S, bool sparse);
 
 }  // namespace i4

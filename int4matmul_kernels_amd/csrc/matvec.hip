@@ -723,7 +723,7 @@ extern "C" int int4mm_matvec(int bits, void* outs, const void* matrix, const voi
     // several batch elements of one row each: one pass over the weights for all of them
     if (B >= 2 && B <= 96 && !tuning(TUNE_NO_SKINNY) &&
         skinny_rows(bits, (h16*)outs, (const uint32_t*)matrix, (const h16*)multiplier, (const h16*)scales,
-                    (const h16*)zeros, B, K, S, g, true, (hipStream_t)stream, (const uint32_t*)sparse_mask))
+                    (const h16*)zeros, B, K, S, g, true, (hipStream_t)stream, (const uint32_t*)sparse_mask, workspace, workspace_bytes))
         return check_launch("matvec");
 
     // Launch shape: strips of 256/lk columns, `waves` waves per workgroup, `upwg`

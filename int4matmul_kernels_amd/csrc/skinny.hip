@@ -38,6 +38,7 @@
 //     y[m, n] += s[n] * (2^24 (accA - accM) - z[n] * 2^20 accM).
 #include "common.h"
 
+#include <algorithm>
 #include <atomic>
 #include <type_traits>
 
@@ -54,6 +55,12 @@ struct SkinnyArgs {
     int group_units;        // group size / 64
     int units_per_wave;
     int accumulate;         // 1: outs = fp16(fp32(outs) + product) (matvec semantics); 0: overwrite
+    // split-K across workgroups (gridDim.z > 1; narrow matrices with a long K): each workgroup takes
+    // `units_per_split` units, stores its fp32 partial tile to `part` and counts itself in; the last one
+    // to arrive adds the partials up in split order and writes the strip
+    int units_per_split;
+    float* part;
+    int* counters;
 };
 
 constexpr int SK_PITCH = 144;                   // bytes between rows of a staged unit (128 + 16: conflict-free)
@@ -173,7 +180,8 @@ __global__ __launch_bounds__(512) void skinny_kernel(SkinnyArgs a) {
     const int j = lane & 15, h = lane >> 4;
     const int col0 = blockIdx.x * STRIP + CW * j;              // first of this lane's CW columns
     const int units = a.K / 64;
-    const int u0 = wave * a.units_per_wave, u1 = min(units, u0 + a.units_per_wave);
+    const int split_lo = blockIdx.z * a.units_per_split, split_hi = min(units, split_lo + a.units_per_split);
+    const int u0 = min(split_hi, split_lo + wave * a.units_per_wave), u1 = min(split_hi, u0 + a.units_per_wave);
     // more than 32 rows: blockIdx.y takes rows 32 y .. 32 y + 31 (each block reads the strip's weights again)
     const int row0 = blockIdx.y * 32;
     const int R = min(32, a.R - row0);
@@ -183,7 +191,9 @@ __global__ __launch_bounds__(512) void skinny_kernel(SkinnyArgs a) {
     // weights and states.  Exponent-mode scales (negative or NaN) anywhere in the
     // strip switch the whole workgroup to the exact per-weight decode.  (The copy
     // runs after the first loads have been issued, under their latency.)
-    const int groups = (units + a.group_units - 1) / a.group_units;
+    // (of the groups that the workgroup's share of K touches: group_lo onwards)
+    const int group_lo = split_lo / a.group_units;
+    const int groups = (split_hi + a.group_units - 1) / a.group_units - group_lo;
     // (16:32: the selector table is allocated statically: its LDS address is a compile-time constant)
     __shared__ __attribute__((aligned(16))) u32x4 lut_table[SPARSE ? 256 : 1];
     const char* lut = reinterpret_cast<const char*>(lut_table);
@@ -215,7 +225,7 @@ __global__ __launch_bounds__(512) void skinny_kernel(SkinnyArgs a) {
         const int n = groups * (STRIP / 2);
         for (int i = t; i < n; i += blockDim.x) {
             const int g = i / (STRIP / 2), c = i % (STRIP / 2);
-            const int64_t at = (int64_t)g * a.S + blockIdx.x * STRIP + 2 * c;
+            const int64_t at = (int64_t)(group_lo + g) * a.S + blockIdx.x * STRIP + 2 * c;
             const uint32_t two = *reinterpret_cast<const uint32_t*>(a.scales + at);
             bad |= !(as_h2(two).x >= (h16)0.0f) || !(as_h2(two).y >= (h16)0.0f);
             sz[i] = two;
@@ -341,7 +351,7 @@ __global__ __launch_bounds__(512) void skinny_kernel(SkinnyArgs a) {
 #pragma unroll
         for (int c = 0; c < CW; ++c) { sc[c] = (h16)0.f; ze[c] = (h16)0.f; }
         auto load_sz = [&](int gi) {
-            const h16* ps = reinterpret_cast<const h16*>(sz) + gi * STRIP + CW * j;
+            const h16* ps = reinterpret_cast<const h16*>(sz) + (gi - group_lo) * STRIP + CW * j;
             const h16* pz = ps + groups * STRIP;
             if constexpr (CW == 4) {
                 const u32x2 s2 = *reinterpret_cast<const u32x2*>(ps), z2 = *reinterpret_cast<const u32x2*>(pz);
@@ -501,6 +511,53 @@ __global__ __launch_bounds__(512) void skinny_kernel(SkinnyArgs a) {
         __syncthreads();
     }
     if (wave == 0) {
+        if (gridDim.z > 1) {
+            // hand-over between the workgroups of a strip: write-through stores of the partial tile
+            // (value v of lane l at (v * 64 + l) * 4), a device-scope counter, and whoever finds all
+            // the others counted reads every partial back in split order -- one summation order
+            // whoever is last -- and goes on to write the strip.  One wave: no barrier involved.
+            constexpr int NV = CW * MT * 4, THROUGH = 17;                 // sc0 | sc1: straight to memory
+            const int tile = blockIdx.y * gridDim.x + blockIdx.x, ks = gridDim.z;
+            char* const slots = reinterpret_cast<char*>(a.part) + (int64_t)tile * ks * (NV * 256);
+            const __amdgpu_buffer_rsrc_t mine = __builtin_amdgcn_make_buffer_rsrc(
+                slots + (int64_t)blockIdx.z * (NV * 256), 0, NV * 256, 0x00020000);
+#pragma unroll
+            for (int c = 0; c < CW; ++c)
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const float v = y[c][mt][e];       // (a bit_cast straight from the vector element reads element 0)
+                        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), mine,
+                                                              (((c * MT + mt) * 4 + e) * 64 + lane) * 4, 0, THROUGH);
+                    }
+            // (the fences keep the compiler from moving the counter update ahead of the stores, or the
+            // loads below ahead of it; the hardware side is the wait for the stores' acknowledgement)
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_s_waitcnt(0);
+            int arrived = 0;
+            if (lane == 0) arrived = __hip_atomic_fetch_add(a.counters + tile, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            arrived = __builtin_amdgcn_readfirstlane(arrived);
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            if (arrived != ks - 1) return;
+            if (lane == 0) __hip_atomic_store(a.counters + tile, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+            for (int c = 0; c < CW; ++c)
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) y[c][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+            for (int sp = 0; sp < ks; ++sp) {
+                const __amdgpu_buffer_rsrc_t theirs = __builtin_amdgcn_make_buffer_rsrc(
+                    slots + (int64_t)sp * (NV * 256), 0, NV * 256, 0x00020000);
+#pragma unroll
+                for (int c = 0; c < CW; ++c)
+#pragma unroll
+                    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            y[c][mt][e] += __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                                theirs, (((c * MT + mt) * 4 + e) * 64 + lane) * 4, 0, THROUGH));
+            }
+        }
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
@@ -520,15 +577,16 @@ __global__ __launch_bounds__(512) void skinny_kernel(SkinnyArgs a) {
 }
 
 template <int BITS, int CW, bool SPARSE>
-static bool launch_skinny(const SkinnyArgs& a, int waves, hipStream_t st) {
+static bool launch_skinny(const SkinnyArgs& a, int waves, int ksplit, hipStream_t st) {
     const int strips = a.S / (16 * CW);
     const int rt = ((a.R > 32 ? 32 : a.R) + 7) / 8;
-    const int groups = (a.K / 64 + a.group_units - 1) / a.group_units;
+    int groups = (a.K / 64 + a.group_units - 1) / a.group_units;
+    if (ksplit > 1) groups = std::min(groups, (a.units_per_split + a.group_units - 1) / a.group_units + 1);
     size_t lds = (size_t)waves * SK_WAVE_LDS + 16 + (size_t)groups * 16 * CW * 4;
     const size_t red = (size_t)(waves / 2) * (rt <= 2 ? 1 : 2) * 16 * 16 * CW * 4;
     if (red > lds) lds = red;
     if (lds > 150 * 1024 - (SPARSE ? 4096 : 0)) return false;      // (16:32: 4 KB of static LDS for the selector table)
-    const dim3 grid(strips, (a.R + 31) / 32), block(waves * 64);
+    const dim3 grid(strips, (a.R + 31) / 32, ksplit), block(waves * 64);
     auto go = [&](auto kernel, int slot) {
         // more than 64 KB of dynamic LDS has to be requested once per kernel and device
         static std::atomic<uint64_t> done[3];
@@ -549,10 +607,52 @@ static bool launch_skinny(const SkinnyArgs& a, int waves, hipStream_t st) {
 }
 
 template <int BITS, bool SPARSE = false>
-static bool launch_skinny_cw(const SkinnyArgs& a, int cw, int waves, hipStream_t st) {
-    if (cw == 4) return launch_skinny<BITS, 4, SPARSE>(a, waves, st);
-    if (cw == 2) return launch_skinny<BITS, 2, SPARSE>(a, waves, st);
-    return launch_skinny<BITS, 1, SPARSE>(a, waves, st);
+static bool launch_skinny_cw(const SkinnyArgs& a, int cw, int waves, int ksplit, hipStream_t st) {
+    if (cw == 4) return launch_skinny<BITS, 4, SPARSE>(a, waves, ksplit, st);
+    if (cw == 2) return launch_skinny<BITS, 2, SPARSE>(a, waves, ksplit, st);
+    return launch_skinny<BITS, 1, SPARSE>(a, waves, ksplit, st);
+}
+
+// Columns per lane of the unsplit kernel: the widest strips (64, 32 or 16 columns) that still give at
+// least 256 workgroups, else at least 128 (narrow strips use half a cache line per packed row).
+static int unsplit_cw(int64_t R, int64_t S, bool sparse) {
+    int cw = 1;
+    const int prefer[4][2] = {{4, 256}, {2, 256}, {4, 128}, {2, 128}};       // {columns per lane, workgroups}
+    for (const auto& c : prefer)
+        if (S % (16 * c[0]) == 0 && S / (16 * c[0]) >= c[1]) { cw = c[0]; break; }
+    // (16:32 with more than 16 rows: four columns per lane would not fit the register file)
+    if (sparse && R > 16 && cw == 4) cw = 2;
+    return cw;
+}
+
+// Split-K plan of the few-row kernel: when even 32-column strips would give fewer than 192 workgroups,
+// 64-column strips with as many workgroups per strip as come closest to one per CU, each with at least
+// six units per wave -- if that makes at least as many workgroups as the unsplit choice of narrower
+// strips (with more than 16 rows, where wide strips matter more: half as many).  `part_bytes`: room for
+// the partial tiles (0: no split).
+struct SkinnySplit { int cw, ksplit; size_t tiles, part_bytes; };
+static SkinnySplit plan_skinny_split(int64_t R, int64_t K, int64_t S, bool sparse) {
+    SkinnySplit p{0, 1, 0, 0};
+    if (S % 64 != 0 || R < 2 || R > 96) return p;
+    const int64_t row_blocks = (R + 31) / 32, units = K / 64;
+    if (S / 32 * row_blocks >= 192) return p;
+    const int cw = sparse && R > 16 ? 2 : 4;
+    const int64_t wgs = S / (16 * cw) * row_blocks;
+    int64_t ks = std::min<int64_t>(256 / wgs, units / (8 * 6));
+    if ((R > 16 ? 2 : 1) * wgs * ks < S / (16 * unsplit_cw(R, S, sparse)) * row_blocks) ks = 1;
+    const int64_t forced = tuning(TUNE_MM_SPLIT);
+    if (forced >= 1) ks = std::min<int64_t>(forced, std::max<int64_t>(1, units / 16));
+    if (ks < 2 || wgs > 1024) return p;
+    p.cw = cw;
+    p.ksplit = (int)ks;
+    p.tiles = (size_t)wgs;
+    p.part_bytes = (size_t)wgs * ks * (cw * 2 * 4 * 256);       // up to 32 rows x 16 cw columns of fp32 per partial
+    return p;
+}
+
+size_t skinny_workspace_bytes(int64_t R, int64_t K, int64_t S, bool sparse) {
+    const SkinnySplit p = plan_skinny_split(R, K, S, sparse);
+    return p.ksplit > 1 ? 4096 + p.part_bytes : 0;
 }
 
 // Product of 2 <= R <= 96 rows with a dense or (sparse_mask != nullptr) 16:32 sparse int4 matrix; beyond that
@@ -560,7 +660,7 @@ static bool launch_skinny_cw(const SkinnyArgs& a, int cw, int waves, hipStream_t
 // uses the general kernels).
 bool skinny_rows(int bits, h16* outs, const uint32_t* matrix, const h16* x, const h16* scales, const h16* zeros,
                  int64_t R, int64_t K, int64_t S, int64_t group_size, bool accumulate, hipStream_t st,
-                 const uint32_t* sparse_mask) {
+                 const uint32_t* sparse_mask, void* workspace, size_t workspace_bytes) {
     if (R < 2 || R > 96 || S % 16 != 0 || K % 64 != 0 || K > (1 << 30) || S > (1 << 28)) return false;
     if (sparse_mask && bits != 4) return false;
     SkinnyArgs a;
@@ -569,25 +669,35 @@ bool skinny_rows(int bits, h16* outs, const uint32_t* matrix, const h16* x, cons
     const int64_t gu = group_size / 64;
     a.group_units = (int)(gu > 0x7FFFFFF ? 0x7FFFFFF : gu);
     a.accumulate = accumulate ? 1 : 0;
-    // widest strips (64, 32 or 16 columns) that still give at least 256 workgroups,
-    // else at least 128 (narrow strips use half a cache line per packed row);
     // four waves split K when there are 256 workgroups (three of them fit a CU) and K
     // is short (each wave should walk a dozen units or more), eight otherwise
-    int cw = 1;
-    const int prefer[4][2] = {{4, 256}, {2, 256}, {4, 128}, {2, 128}};       // {columns per lane, workgroups}
-    for (const auto& c : prefer)
-        if (S % (16 * c[0]) == 0 && S / (16 * c[0]) >= c[1]) { cw = c[0]; break; }
-    // (16:32 with more than 16 rows: four columns per lane would not fit the register file)
-    if (sparse_mask && R > 16 && cw == 4) cw = 2;
+    int cw = unsplit_cw(R, S, sparse_mask != nullptr);
     const int units = (int)(K / 64);
     int waves = (int)tuning(TUNE_MV_WAVES);
     if (waves != 2 && waves != 4 && waves != 8) waves = S / (16 * cw) >= 256 && units < 160 ? 4 : 8;
     while (waves > 1 && units < 2 * waves) waves >>= 1;
-    a.units_per_wave = (units + waves - 1) / waves;
-    if (sparse_mask) return launch_skinny_cw<4, true>(a, cw, waves, st);
-    if (bits == 4) return launch_skinny_cw<4>(a, cw, waves, st);
-    if (bits == 3) return launch_skinny_cw<3>(a, cw, waves, st);
-    return launch_skinny_cw<2>(a, cw, waves, st);
+    auto launch = [&](int cw_, int waves_, int ksplit_) {
+        a.units_per_wave = (a.units_per_split + waves_ - 1) / waves_;
+        if (sparse_mask) return launch_skinny_cw<4, true>(a, cw_, waves_, ksplit_, st);
+        if (bits == 4) return launch_skinny_cw<4>(a, cw_, waves_, ksplit_, st);
+        if (bits == 3) return launch_skinny_cw<3>(a, cw_, waves_, ksplit_, st);
+        return launch_skinny_cw<2>(a, cw_, waves_, ksplit_, st);
+    };
+    // split-K across workgroups where the plan asks for it and the workspace (behind the matvec's part:
+    // one page of per-strip counters, then the partial tiles) has room
+    a.part = nullptr;
+    a.counters = nullptr;
+    const SkinnySplit sp = plan_skinny_split(R, K, S, sparse_mask != nullptr);
+    const size_t base = int4mm_workspace_bytes(S);
+    if (sp.ksplit > 1 && workspace != nullptr && workspace_bytes >= base + 4096 + sp.part_bytes) {
+        a.units_per_split = (units + sp.ksplit - 1) / sp.ksplit;
+        a.counters = reinterpret_cast<int*>(static_cast<char*>(workspace) + base);
+        a.part = reinterpret_cast<float*>(static_cast<char*>(workspace) + base + 4096);
+        const int ksplit = (units + a.units_per_split - 1) / a.units_per_split;          // no empty split
+        if (launch(sp.cw, 8, ksplit)) return true;
+    }
+    a.units_per_split = units;
+    return launch(cw, waves, 1);
 }
 
 }  // namespace i4

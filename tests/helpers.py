@@ -26,8 +26,8 @@ def run_capi(p, d, kind, outs_init=None):
     B, M, S = p["B"], p["M"], p["S"]
     outs = torch.zeros((B, M, S), dtype=torch.float16, device=DEV) if outs_init is None \
         else t(outs_init).clone()
-    # (the matmul workspace is the matvec's plus room for split-K partial tiles where the shape wants them)
-    ws = capi.new_workspace(S) if kind == "vec" else capi.new_matmul_workspace(B, M, p["K"], S, d["mask"] is not None)
+    # (the matvec's workspace plus room for split-K partial tiles where the shape wants them)
+    ws = capi.new_matmul_workspace(B, M, p["K"], S, d["mask"] is not None)
     fn = capi.matvec if kind == "vec" else capi.matmul
     fn(p["bits"], outs, d["matrix"], d["states"], d["scales"], d["zeros"], p["group_size"],
        d["mask"], ws)

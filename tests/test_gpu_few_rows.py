@@ -162,3 +162,35 @@ def test_few_rows_sparse_degenerate_known_answer(H):
 def test_few_rows_sparse_full_size(H):
     p = O.make_problem(bits=4, K=5120, S=20480, M=8, group_size=64, sparse=True, seed=4)
     _check(H, p, "mtx")
+
+
+# ---- long K against a narrow matrix: the strips are split along K across workgroups
+@pytest.mark.parametrize("bits,sparse", [(4, False), (3, False), (2, False), (4, True)])
+@pytest.mark.parametrize("M,K,S,g", [(8, 16384, 256, 128), (40, 8192, 128, 64), (2, 12288, 512, -1), (17, 6144, 192, 128)])
+def test_few_rows_split_k(H, bits, sparse, M, K, S, g):
+    capi = H.capi
+    p = _problem(bits, K=K, S=S, M=M, group_size=g, seed=M + S, sparse=sparse)
+    assert capi.matmul_workspace_bytes(1, M, K, S, sparse) > capi.lib().int4mm_workspace_bytes(S), "shape should split"
+    d = H.dev_problem(p)
+    exact, f32 = H.oracles(p)
+    outs = []
+    ws = capi.new_matmul_workspace(1, M, K, S, sparse)
+    for _ in range(3):                                   # one workspace: the counters must come back to zero
+        o = torch.full((1, M, S), -5.0, dtype=torch.float16, device="cuda")
+        capi.matmul(bits, o, d["matrix"], d["states"], d["scales"], d["zeros"], g, d["mask"], ws)
+        torch.cuda.synchronize()
+        outs.append(o.cpu().numpy())
+    H.assert_product_close(outs[0], exact, f32, kind="vec")
+    assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[0], outs[2])
+    capi.tune(6, 1)                                      # unsplit
+    try:
+        ref = H.run_capi(p, d, "mtx")
+    finally:
+        capi.tune(6, 0)
+    assert O.max_rel_error(ref.astype(np.float64), outs[0]) < H.TOL_EXACT
+
+
+def test_few_rows_split_k_matvec_entry_accumulates(H):
+    p = _problem(4, K=16384, S=256, M=1, B=6, group_size=128, seed=77)
+    prior = np.random.default_rng(1).standard_normal((6, 1, 256)).astype(np.float16)
+    _check(H, p, "vec", prior=prior)
