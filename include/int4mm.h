@@ -96,7 +96,10 @@ typedef struct int4mm_shape {
  * out_size <= `max_out_size` (partial sums and arrival counters of the split-K
  * finish).  The buffer must be zero-filled once before its first use (e.g. with
  * int4mm_workspace_init); the kernels leave it zeroed where it must be zero.
- * Calls that share one workspace must not overlap in time. */
+ * Calls that share one workspace must not overlap in time.  Calls of different
+ * shapes may share one: its layout depends on its size alone (the lower half is
+ * kept zero -- hand-over slots, arrival counters -- and the upper half is scratch
+ * for partial tiles), so always pass the size the buffer was zero-filled with. */
 INT4MM_API size_t int4mm_workspace_bytes(int64_t max_out_size);
 INT4MM_API int int4mm_workspace_init(void* workspace, size_t workspace_bytes, void* stream);
 

@@ -94,11 +94,9 @@ int int4mm_tune(int key, int64_t value) {
     return INT4MM_OK;
 }
 
-// hand-over slots of the matvec: up to 32 K-splits x out_size x {fp32, flag}
+// the matvec's slots and the counter page in the half that is kept zero; as much again above it
 size_t int4mm_workspace_bytes(int64_t max_out_size) {
-    if (max_out_size < 0) max_out_size = 0;
-    size_t s = (size_t)((max_out_size + 255) / 256 * 256);
-    return 4096 + s * 8 * 32;
+    return 2 * (matvec_slots_bytes(max_out_size) + 4096);
 }
 
 int int4mm_workspace_init(void* workspace, size_t workspace_bytes, void* stream) {

@@ -95,7 +95,34 @@ enum TuneKey { TUNE_MV_WAVES = 0, TUNE_MV_UNITS = 1, TUNE_MV_LK = 2, TUNE_MM_VAR
 bool skinny_rows(int bits, _Float16* outs, const uint32_t* matrix, const _Float16* x, const _Float16* scales,
                  const _Float16* zeros, int64_t R, int64_t K, int64_t S, int64_t group_size, bool accumulate,
                  hipStream_t st, const uint32_t* sparse_mask, void* workspace, size_t workspace_bytes);
-// room the few-row kernel wants behind the matvec's part of the workspace to split K across workgroups (0: none)
+// bytes of partial tiles with which the few-row kernel splits K across workgroups (0: no split)
 size_t skinny_workspace_bytes(int64_t R, int64_t K, int64_t S, bool sparse);
+
+// Layout of a caller's workspace, a function of its size alone so that calls with different shapes may
+// share one buffer.  The lower half (down to a page boundary) is kept zero between calls: the matvec's
+// hand-over slots from byte 0 and, in its last page, the arrival counters of the split-K kernels.  The
+// upper half is scratch for partial tiles; no call relies on what it holds.
+struct WorkspaceParts {
+    char* counters;           // one page (nullptr: the workspace has no room for it)
+    char* scratch;
+    size_t slots_bytes;       // room for the matvec's slots, below the counters
+    size_t scratch_bytes;
+};
+inline WorkspaceParts workspace_parts(void* workspace, size_t bytes) {
+    WorkspaceParts p{nullptr, nullptr, 0, 0};
+    const size_t kept_zero = (bytes / 2) & ~size_t(4095);
+    if (workspace == nullptr || kept_zero < 8192) return p;
+    p.counters = static_cast<char*>(workspace) + kept_zero - 4096;
+    p.scratch = static_cast<char*>(workspace) + kept_zero;
+    p.slots_bytes = kept_zero - 4096;
+    p.scratch_bytes = bytes - kept_zero;
+    return p;
+}
+// the matvec's hand-over slots: up to 32 K-splits x out_size (in 256s) x {fp32, flag}
+inline size_t matvec_slots_bytes(int64_t out_size) {
+    if (out_size < 0) out_size = 0;
+    return 4096 + (size_t)((out_size + 255) / 256 * 256) * 8 * 32;
+}
+inline size_t round_to_page(size_t n) { return (n + 4095) & ~size_t(4095); }
 
 }  // namespace i4

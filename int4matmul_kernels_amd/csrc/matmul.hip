@@ -962,16 +962,16 @@ static void launch(MatmulArgs a, int64_t B, hipStream_t st, void* workspace, siz
         else if (a.M > 512 && a.S >= 256) variant = 3;
         else variant = 1;
     }
-    // split-K where the plan asks for it and the caller's workspace has room (it then holds, behind
-    // the matvec's part, one page of per-tile counters and the partial tiles)
+    // split-K where the plan asks for it and the scratch half of the caller's workspace has room for
+    // the partial tiles (the per-tile counters sit in the last page of the half that is kept zero)
     if ((SPARSE && (variant == 6 || variant == 9)) || (!SPARSE && variant == 5)) {
         const SplitPlan sp = plan_split(SPARSE, B, a.M, a.K, a.S);
-        const size_t base = int4mm_workspace_bytes(a.S);
-        if (sp.ksplit > 1 && workspace != nullptr &&
-            workspace_bytes >= base + 4096 + (size_t)(sp.tiles * sp.ksplit * sp.tile_bytes)) {
+        const WorkspaceParts ws = workspace_parts(workspace, workspace_bytes);
+        if (sp.ksplit > 1 && ws.counters != nullptr && sp.tiles <= 1024 &&
+            ws.scratch_bytes >= (size_t)(sp.tiles * sp.ksplit * sp.tile_bytes)) {
             a.ksplit = sp.ksplit;
-            a.counters = reinterpret_cast<int*>(static_cast<char*>(workspace) + base);
-            a.part = reinterpret_cast<float*>(static_cast<char*>(workspace) + base + 4096);
+            a.counters = reinterpret_cast<int*>(ws.counters);
+            a.part = reinterpret_cast<float*>(ws.scratch);
         }
     }
     if (variant == 1) launch_tile<BITS, SPARSE, 128, 128, 64, 64>(a, B, st);
@@ -1029,15 +1029,15 @@ extern "C" int int4mm_matmul(int bits, void* outs, const void* matrix, const voi
     return check_launch("matmul");
 }
 
-// Workspace with which int4mm_matmul may split K for this shape: the matvec's part, one page of
-// counters and the partial tiles.  A smaller workspace is not an error: the product then runs unsplit.
+// Workspace with which int4mm_matmul may split K for this shape: what the matvec needs, plus room for
+// the partial tiles in the scratch half.  A smaller workspace is not an error: the product then runs unsplit.
 extern "C" size_t int4mm_matmul_workspace_bytes(const int4mm_shape* shape, int sparse) {
     if (shape == nullptr) return 0;
     const int64_t B = shape->batch, M = shape->seq_len, K = shape->in_size, S = shape->out_size;
     size_t need = int4mm_workspace_bytes(S);
     if (B <= 0 || M <= 0 || K < 64 || S < 128) return need;
-    if (B * M <= 96) return need + skinny_workspace_bytes(B * M, K, S, sparse != 0);
+    if (B * M <= 96) return need + 2 * round_to_page(skinny_workspace_bytes(B * M, K, S, sparse != 0));
     const SplitPlan sp = plan_split(sparse != 0, B, M, K, S);
-    if (sp.ksplit > 1) need += 4096 + (size_t)(sp.tiles * sp.ksplit * sp.tile_bytes);
+    if (sp.ksplit > 1) need += 2 * round_to_page((size_t)(sp.tiles * sp.ksplit * sp.tile_bytes));
     return need;
 }

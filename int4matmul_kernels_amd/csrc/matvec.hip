@@ -755,7 +755,7 @@ extern "C" int int4mm_matvec(int bits, void* outs, const void* matrix, const voi
     }
     if (waves * lk > upwg) waves = (upwg + lk - 1) / lk;    // no idle waves
     if (upwg > MV_MAX_UNITS_WG) return INT4MM_ERR_SHAPE;
-    if (splits > 1 && (workspace == nullptr || workspace_bytes < int4mm_workspace_bytes(S)))
+    if (splits > 1 && workspace_parts(workspace, workspace_bytes).slots_bytes < matvec_slots_bytes(S))
         return INT4MM_ERR_WORKSPACE;
     // software prefetch only pays when lane groups walk several units
     const bool pf = upwg >= 3 * waves * lk && tuning(TUNE_MV_NOPF) == 0;

@@ -652,7 +652,7 @@ static SkinnySplit plan_skinny_split(int64_t R, int64_t K, int64_t S, bool spars
 
 size_t skinny_workspace_bytes(int64_t R, int64_t K, int64_t S, bool sparse) {
     const SkinnySplit p = plan_skinny_split(R, K, S, sparse);
-    return p.ksplit > 1 ? 4096 + p.part_bytes : 0;
+    return p.ksplit > 1 ? p.part_bytes : 0;
 }
 
 // Product of 2 <= R <= 96 rows with a dense or (sparse_mask != nullptr) 16:32 sparse int4 matrix; beyond that
@@ -683,16 +683,16 @@ bool skinny_rows(int bits, h16* outs, const uint32_t* matrix, const h16* x, cons
         if (bits == 3) return launch_skinny_cw<3>(a, cw_, waves_, ksplit_, st);
         return launch_skinny_cw<2>(a, cw_, waves_, ksplit_, st);
     };
-    // split-K across workgroups where the plan asks for it and the workspace (behind the matvec's part:
-    // one page of per-strip counters, then the partial tiles) has room
+    // split-K across workgroups where the plan asks for it and the scratch half of the workspace has room
+    // for the partial tiles (per-strip counters: last page of the half that is kept zero)
     a.part = nullptr;
     a.counters = nullptr;
     const SkinnySplit sp = plan_skinny_split(R, K, S, sparse_mask != nullptr);
-    const size_t base = int4mm_workspace_bytes(S);
-    if (sp.ksplit > 1 && workspace != nullptr && workspace_bytes >= base + 4096 + sp.part_bytes) {
+    const WorkspaceParts ws = workspace_parts(workspace, workspace_bytes);
+    if (sp.ksplit > 1 && ws.counters != nullptr && ws.scratch_bytes >= sp.part_bytes) {
         a.units_per_split = (units + sp.ksplit - 1) / sp.ksplit;
-        a.counters = reinterpret_cast<int*>(static_cast<char*>(workspace) + base);
-        a.part = reinterpret_cast<float*>(static_cast<char*>(workspace) + base + 4096);
+        a.counters = reinterpret_cast<int*>(ws.counters);
+        a.part = reinterpret_cast<float*>(ws.scratch);
         const int ksplit = (units + a.units_per_split - 1) / a.units_per_split;          // no empty split
         if (launch(sp.cw, 8, ksplit)) return true;
     }

@@ -65,8 +65,32 @@ def test_split_k_repeated_calls_share_a_workspace(H, bits, sparse):
         assert np.array_equal(r, results[0])              # the sum has one order whoever arrives last
     exact, f32 = H.oracles(p)
     H.assert_product_close(results[0], exact, f32, kind="mtx")
-    base = capi.lib().int4mm_workspace_bytes(512)
-    assert int(ws[base:base + 4096].to(torch.int32).sum()) == 0    # the counters are back to zero
+    kept_zero = (ws.numel() // 2) & ~4095
+    assert int(ws[:kept_zero].to(torch.int32).sum()) == 0         # counters and slots are back to zero
+    assert int(ws[kept_zero:].to(torch.int32).sum()) != 0         # (the partial tiles were there)
+
+
+def test_one_workspace_shared_by_calls_of_different_shapes(H):
+    """The layout of a workspace depends on its size alone: split matmuls, split few-row products
+    and matvecs of different widths may take turns on one buffer."""
+    capi = H.capi
+    shapes = [("mtx", 4, False, 256, 2048, 512, 128), ("vec", 4, False, 1, 4096, 1024, 128),
+              ("mtx", 4, False, 8, 16384, 256, 128), ("vec", 4, True, 1, 2048, 2048, 64),
+              ("mtx", 4, True, 256, 2048, 256, 64), ("mtx", 3, False, 40, 8192, 128, 64),
+              ("vec", 2, False, 1, 8192, 192, 128), ("mtx", 4, False, 200, 1536, 768, 64)]
+    need = max(capi.matmul_workspace_bytes(1, M, K, S, sparse) for _, _, sparse, M, K, S, _ in shapes)
+    ws = torch.zeros(need, dtype=torch.uint8, device="cuda")
+    cases = []
+    for kind, bits, sparse, M, K, S, g in shapes:
+        p = _problem(bits, sparse, K=K, S=S, M=M, group_size=g, seed=K + S)
+        cases.append((kind, bits, g, p, H.dev_problem(p), H.oracles(p)))
+    for _ in range(2):
+        for kind, bits, g, p, d, (exact, f32) in cases:
+            outs = torch.zeros((1, p["M"], p["S"]), dtype=torch.float16, device="cuda")
+            fn = capi.matmul if kind == "mtx" else capi.matvec
+            fn(bits, outs, d["matrix"], d["states"], d["scales"], d["zeros"], g, d["mask"], ws)
+            torch.cuda.synchronize()
+            H.assert_product_close(outs.cpu().numpy(), exact, f32, kind="vec" if p["M"] <= 96 else "mtx")
 
 
 def test_split_k_needs_room_in_the_workspace(H):
@@ -98,3 +122,19 @@ def test_split_k_through_the_extension(H, bits, sparse):
     exact, f32 = H.oracles(p)
     for _ in range(2):
         H.assert_product_close(H.run_ext(p, d), exact, f32, kind="mtx")
+
+
+def test_extension_workspace_survives_changing_shapes(H):
+    """The extension keeps one workspace per stream and lets it grow: products of different widths, split or
+    not, follow each other through `quant_matmul`."""
+    shapes = [(4, False, 16, 8192, 1024, 128), (4, False, 32, 16384, 256, 128), (4, False, 64, 8192, 512, 128),
+              (4, True, 8, 8192, 1024, 64), (4, False, 1, 4096, 2048, 128), (4, False, 256, 2048, 512, 128),
+              (3, False, 1, 4096, 512, 128), (4, False, 16, 8192, 1024, 128)]
+    cases = []
+    for bits, sparse, M, K, S, g in shapes:
+        p = _problem(bits, sparse, K=K, S=S, M=M, group_size=g, seed=K + S + M)
+        cases.append((p, H.dev_problem(p), H.oracles(p)))
+    for _ in range(2):
+        for p, d, (exact, f32) in cases:
+            got = H.run_ext(p, d)
+            H.assert_product_close(got, exact, f32, kind="vec" if p["M"] <= 96 else "mtx")
