@@ -49,6 +49,9 @@ struct MatmulArgs {
     int ksplit;
     float* part;
     int* counters;
+    // tiles (in grid order) before `split_from` are not split: a grid whose last round would fill
+    // at most half of the GPU splits only the tiles of that round
+    int split_from;
 };
 
 // Raw packed data of one (32-row block, column) cell
@@ -398,7 +401,8 @@ constexpr int P_STAGES = 3;
 // finishing the step alone.
 template <int BITS, bool SPARSE, int TM, int NW, bool PING, bool SPLIT>
 __device__ __forceinline__ void pipe_tile(const MatmulArgs& a, const int m0, const int s0, const h16* x,
-                                          h16* outs, h16* As, h16* Bs, uint32_t* lut, const int tile, const int split) {
+                                          h16* outs, h16* As, h16* Bs, uint32_t* lut, const int tile, const int split,
+                                          const int nsplit) {
     constexpr int BM = TM * 64, BN = NW * 64, WM = TM * 32, WN = 64, TN = 2, T = 2 * NW * 64;
     constexpr int A_STAGE = BM * PK, B_STAGE = PK * BN;            // halves per stage
     constexpr int A_ROWS = T / 4;                                  // rows covered by one 16-byte load per thread
@@ -562,7 +566,7 @@ __device__ __forceinline__ void pipe_tile(const MatmulArgs& a, const int m0, con
 
     // K steps kt0 .. last of the matrix belong to this workgroup (all of them unless SPLIT)
     const int ksteps = a.K / PK;
-    const int per_split = SPLIT ? (ksteps + a.ksplit - 1) / a.ksplit : ksteps;
+    const int per_split = SPLIT ? (ksteps + nsplit - 1) / nsplit : ksteps;
     const int kt0 = SPLIT ? split * per_split : 0;
     const int ktiles = SPLIT ? min(ksteps, kt0 + per_split) - kt0 : ksteps;
     const int last = kt0 + ktiles - 1;
@@ -778,16 +782,17 @@ __device__ __forceinline__ void pipe_tile(const MatmulArgs& a, const int m0, con
             __syncthreads();
         }
     }
-    if constexpr (SPLIT) {
+    if (SPLIT && nsplit > 1) {
         // Every workgroup of the tile stores its partial accumulators (16 bytes per lane and
         // store: register group g of thread t at (g * T + t) * 16 -- whole cache lines per wave)
         // and then counts itself in; whoever finds all the others counted adds the partials up
         // in split order (its own included, from memory: the sum has one order whoever is
         // last) and writes the tile.  Stores and loads go straight through to memory
         // (system-scope cache policy), the counter is a device-scope atomic: no cache-wide
-        // fence, no waiting.
-        constexpr int GROUPS = TM * TN * 4, SLOT_BYTES = BM * BN * 4, THROUGH = 17;      // sc0 | sc1
-        char* const slots = reinterpret_cast<char*>(a.part) + (int64_t)tile * a.ksplit * SLOT_BYTES;
+        // fence, no waiting.  (Two workgroups per tile: the last one adds the other's partial to
+        // its own registers -- a sum of two terms has one value in either order.)
+        constexpr int SLOT_BYTES = BM * BN * 4, THROUGH = 17;      // sc0 | sc1
+        char* const slots = reinterpret_cast<char*>(a.part) + (int64_t)tile * nsplit * SLOT_BYTES;
         const __amdgpu_buffer_rsrc_t mine = __builtin_amdgcn_make_buffer_rsrc(
             slots + (int64_t)split * SLOT_BYTES, 0, SLOT_BYTES, RSRC_FLAGS);
 #pragma unroll
@@ -804,15 +809,17 @@ __device__ __forceinline__ void pipe_tile(const MatmulArgs& a, const int m0, con
         __syncthreads();
         if (t == 0) *flag = __hip_atomic_fetch_add(a.counters + tile, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __syncthreads();
-        if (*flag != a.ksplit - 1) return;
+        if (*flag != nsplit - 1) return;
         if (t == 0) __hip_atomic_store(a.counters + tile, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // clean for the next call
+        if (nsplit > 2) {
 #pragma unroll
-        for (int i = 0; i < TM; ++i)
+            for (int i = 0; i < TM; ++i)
 #pragma unroll
-            for (int j = 0; j < TN; ++j)
+                for (int j = 0; j < TN; ++j)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-        for (int sp = 0; sp < a.ksplit; ++sp) {
+                    for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+        }
+        for (int sp = nsplit > 2 ? 0 : 1 - split; sp < (nsplit > 2 ? nsplit : 2 - split); ++sp) {
             const __amdgpu_buffer_rsrc_t theirs = __builtin_amdgcn_make_buffer_rsrc(
                 slots + (int64_t)sp * SLOT_BYTES, 0, SLOT_BYTES, RSRC_FLAGS);
 #pragma unroll
@@ -827,7 +834,6 @@ __device__ __forceinline__ void pipe_tile(const MatmulArgs& a, const int m0, con
                         for (int e = 0; e < 4; ++e) acc[i][j][4 * q + e] += v[e];
                     }
         }
-        (void)GROUPS;
     }
 #pragma unroll
     for (int i = 0; i < TM; ++i)
@@ -848,10 +854,19 @@ __global__ __launch_bounds__(NW * 128, NW == 2 ? 2 : 1) void matmul_kernel_pipe(
     __shared__ __attribute__((aligned(16))) h16 As[P_STAGES * BM * PK];
     __shared__ __attribute__((aligned(16))) h16 Bs[P_STAGES * PK * BN];
     __shared__ __attribute__((aligned(16))) uint32_t Lut[SPARSE ? SPARSE_LUT_WORDS : 4];
-    // (split-K: the workgroups of a tile are neighbours in the grid, so they run at about the same time)
-    const int split = SPLIT ? (int)blockIdx.x % a.ksplit : 0;
-    int bid = SPLIT ? (int)blockIdx.x / a.ksplit : (int)blockIdx.x;
+    // (split-K: the workgroups of a tile are neighbours in the grid, so they run at about the same time;
+    // the tiles before `split_from` are whole)
     const int total = a.tiles_m * a.tiles_n;
+    int bid = blockIdx.x, split = 0, nsplit = 1, slot = 0;
+    if constexpr (SPLIT) {
+        const int v = (int)blockIdx.x - a.split_from;
+        if (v >= 0) {
+            bid = a.split_from + v / a.ksplit;
+            split = v % a.ksplit;
+            nsplit = a.ksplit;
+            slot = (int)blockIdx.z * (total - a.split_from) + v / a.ksplit;       // counter and partial tiles
+        }
+    }
     int tile_m, tile_n;
     if (total % 8 == 0) {
         // XCD-aware numbering: workgroups are dealt round-robin to the 8 XCDs (each
@@ -874,21 +889,19 @@ __global__ __launch_bounds__(NW * 128, NW == 2 ? 2 : 1) void matmul_kernel_pipe(
     }
     const int64_t boff = blockIdx.z;
     pipe_tile<BITS, SPARSE, TM, NW, PING, SPLIT>(a, tile_m * BM, tile_n * BN, a.x + boff * a.M * (int64_t)a.K,
-                                          a.outs + boff * a.M * (int64_t)a.S, As, Bs, Lut,
-                                          ((int)boff * a.tiles_n + tile_n) * a.tiles_m + tile_m, split);
+                                          a.outs + boff * a.M * (int64_t)a.S, As, Bs, Lut, slot, split, nsplit);
 }
 
 template <int BITS, bool SPARSE, int NW, int TM = 4, bool PING = false>
 static void launch_pipe(MatmulArgs a, int64_t B, hipStream_t st) {
     a.tiles_m = (a.M + TM * 64 - 1) / (TM * 64);
     a.tiles_n = a.S / (NW * 64);
-    const dim3 grid(a.tiles_m * a.tiles_n * a.ksplit, 1, (unsigned)B), block(NW * 128);
+    const int total = a.tiles_m * a.tiles_n;
+    const dim3 grid(a.split_from + (total - a.split_from) * a.ksplit, 1, (unsigned)B), block(NW * 128);
     a.by_columns = a.tiles_n % 8 == 0;
-    if constexpr (!PING) {
-        if (a.ksplit > 1) {
-            hipLaunchKernelGGL((matmul_kernel_pipe<BITS, SPARSE, NW, TM, false, true>), grid, block, 0, st, a);
-            return;
-        }
+    if (a.ksplit > 1) {
+        hipLaunchKernelGGL((matmul_kernel_pipe<BITS, SPARSE, NW, TM, PING, true>), grid, block, 0, st, a);
+        return;
     }
     hipLaunchKernelGGL((matmul_kernel_pipe<BITS, SPARSE, NW, TM, PING, false>), grid, block, 0, st, a);
 }
@@ -918,6 +931,20 @@ static SplitPlan plan_split(bool sparse, int64_t B, int64_t M, int64_t K, int64_
     if (best < 2) return none;
     p.ksplit = (int)best;
     return p;
+}
+
+// ---- split of the last round.  256 x 256 tiles run one per CU, in rounds of 256; when the last round
+// would fill at most half of the GPU, its tiles -- and only they -- are split along K over as many
+// workgroups as fit the GPU once (at least 16 K steps each).
+struct TailPlan { int ksplit; int64_t split_from, tiles; };
+static TailPlan plan_tail(int64_t B, int64_t M, int64_t K, int64_t S) {
+    const TailPlan none{1, 0, 0};
+    if (B != 1 || S % 256 != 0 || tuning(TUNE_MM_TAIL) == 1) return none;
+    const int64_t total = (M + 255) / 256 * (S / 256), tail = total % 256;
+    if (total <= 256 || tail == 0 || tail > 128) return none;
+    const int64_t ks = std::min<int64_t>({256 / tail, 8, K / 32 / 16});
+    if (ks < 2 || tail * ks * (256 * 256 * 4) > MM_SPLIT_MAX_BYTES) return none;
+    return TailPlan{(int)ks, total - tail, tail};
 }
 
 template <int BITS, bool SPARSE, int BM, int BN, int WM, int WN>
@@ -953,10 +980,16 @@ static void launch(MatmulArgs a, int64_t B, hipStream_t st, void* workspace, siz
     const bool pipe4_ok = m_ok && a.S % 256 == 0;
     if (variant != 1 && variant != 3 && variant != 5 && variant != 6 && variant != 9) variant = 0;
     if ((variant == 5 && !pipe2_ok) || ((variant == 6 || variant == 9) && !pipe4_ok)) variant = 0;
+    // (a last round of large tiles that fills at most half of the GPU is split along K when the
+    // workspace has room for its partial tiles: better than small tiles then)
+    const TailPlan tp = plan_tail(B, a.M, a.K, a.S);
+    const WorkspaceParts wsp = workspace_parts(workspace, workspace_bytes);
+    const bool tail_ok = pipe4_ok && tp.ksplit > 1 && wsp.counters != nullptr &&
+                         wsp.scratch_bytes >= (size_t)(tp.tiles * tp.ksplit * (256 * 256 * 4));
     if (variant == 0) {
         const int64_t tiles4 = m_pad / 256 * (a.S / 256) * B;
         const int64_t last = tiles4 % 256;
-        const bool small_better = tiles4 <= 128 || (tiles4 > 256 && tiles4 < 512 && last > 0 && last <= 96);
+        const bool small_better = tiles4 <= 128 || (!tail_ok && tiles4 > 256 && tiles4 < 512 && last > 0 && last <= 96);
         if (pipe4_ok && (SPARSE || !pipe2_ok || !small_better)) variant = 6;
         else if (pipe2_ok) variant = 5;
         else if (a.M > 512 && a.S >= 256) variant = 3;
@@ -973,6 +1006,12 @@ static void launch(MatmulArgs a, int64_t B, hipStream_t st, void* workspace, siz
             a.counters = reinterpret_cast<int*>(ws.counters);
             a.part = reinterpret_cast<float*>(ws.scratch);
         }
+    }
+    if (a.ksplit == 1 && (variant == 6 || variant == 9) && tail_ok) {
+        a.ksplit = tp.ksplit;
+        a.split_from = (int)tp.split_from;
+        a.counters = reinterpret_cast<int*>(wsp.counters);
+        a.part = reinterpret_cast<float*>(wsp.scratch);
     }
     if (variant == 1) launch_tile<BITS, SPARSE, 128, 128, 64, 64>(a, B, st);
     else if (variant == 3) launch_tile<BITS, SPARSE, 128, 256, 128, 64>(a, B, st);
@@ -1019,6 +1058,7 @@ extern "C" int int4mm_matmul(int bits, void* outs, const void* matrix, const voi
     a.tiles_m = a.tiles_n = 0;
     a.by_columns = 0;
     a.ksplit = 1;
+    a.split_from = 0;
     a.part = nullptr;
     a.counters = nullptr;
 
@@ -1039,5 +1079,7 @@ extern "C" size_t int4mm_matmul_workspace_bytes(const int4mm_shape* shape, int s
     if (B * M <= 96) return need + 2 * round_to_page(skinny_workspace_bytes(B * M, K, S, sparse != 0));
     const SplitPlan sp = plan_split(sparse != 0, B, M, K, S);
     if (sp.ksplit > 1) need += 2 * round_to_page((size_t)(sp.tiles * sp.ksplit * sp.tile_bytes));
+    const TailPlan tp = plan_tail(B, M, K, S);
+    if (sp.ksplit == 1 && tp.ksplit > 1) need += 2 * round_to_page((size_t)(tp.tiles * tp.ksplit * (256 * 256 * 4)));
     return need;
 }

@@ -138,3 +138,38 @@ def test_extension_workspace_survives_changing_shapes(H):
         for p, d, (exact, f32) in cases:
             got = H.run_ext(p, d)
             H.assert_product_close(got, exact, f32, kind="vec" if p["M"] <= 96 else "mtx")
+
+
+# ---- grids of 256 x 256 tiles whose last round of 256 fills at most half of the GPU: only the tiles of
+# that round are split along K (tuning key 7 = 1 switches it off)
+@pytest.mark.parametrize("bits,sparse", FORMATS)
+@pytest.mark.parametrize("M,K,S,g", [(512, 1024, 33280, 128),        # 260 tiles: 4 split in two
+                                     (2200, 2048, 7424, 64)])        # 261 tiles: 5 split in four
+def test_tail_split_matches_oracle_and_unsplit(H, bits, sparse, M, K, S, g):
+    capi = H.capi
+    p = _problem(bits, sparse, K=K, S=S, M=M, group_size=g, seed=M + K + 1)
+    capi.tune(7, 1)
+    try:
+        plain_bytes = capi.matmul_workspace_bytes(1, M, K, S, sparse)
+    finally:
+        capi.tune(7, 0)
+    assert capi.matmul_workspace_bytes(1, M, K, S, sparse) > plain_bytes, "shape should split its last round"
+    d = H.dev_problem(p)
+    exact, f32 = H.oracles(p)
+    ws = capi.new_matmul_workspace(1, M, K, S, sparse)
+    runs = []
+    for _ in range(3):                                    # one workspace: the counters come back to zero
+        outs = torch.full((1, M, S), 3.0, dtype=torch.float16, device="cuda")
+        capi.matmul(bits, outs, d["matrix"], d["states"], d["scales"], d["zeros"], g, d["mask"], ws)
+        torch.cuda.synchronize()
+        runs.append(outs.cpu().numpy())
+    H.assert_product_close(runs[0], exact, f32, kind="mtx")
+    assert np.array_equal(runs[0], runs[1]) and np.array_equal(runs[0], runs[2])
+    capi.tune(7, 1)
+    try:
+        ref = H.run_capi(p, d, "mtx")
+    finally:
+        capi.tune(7, 0)
+    assert O.max_rel_error(ref.astype(np.float64), runs[0]) < H.TOL_EXACT
+    # the tiles that were not split are bit-identical to the plain run's
+    assert np.array_equal(ref[:, :256, :256], runs[0][:, :256, :256])
