@@ -88,7 +88,8 @@ int int4mm_abi_version(void) { return 1; }
 // 2 = matvec lane groups per wave (1, 2 or 4), 3 = matmul kernel variant,
 // 4 = matvec: 1 disables the software prefetch, 5 = 1 disables the few-row kernel,
 // 6 = matmul split-K factor (1 = never, 2..8 = forced where the shape allows a split),
-// 7 = 1: the tiles of a matmul's last, partly filled round are not split.
+// 7 = 1: the tiles of a matmul's last, partly filled round are not split,
+// 8 = 1: 33 .. 96 rows take the few-row kernel whose waves stage their own states.
 int int4mm_tune(int key, int64_t value) {
     if (key < 0 || key >= TUNE_COUNT) return INT4MM_ERR_SHAPE;
     g_tuning[key].store(value);

@@ -61,6 +61,7 @@ struct SkinnyArgs {
     int units_per_split;
     float* part;
     int* counters;
+    int block_rows;         // wide kernel: rows of states per workgroup (blockIdx.y), a multiple of 16
 };
 
 constexpr int SK_PITCH = 144;                   // bytes between rows of a staged unit (128 + 16: conflict-free)
@@ -576,6 +577,313 @@ __global__ __launch_bounds__(512) void skinny_kernel(SkinnyArgs a) {
     }
 }
 
+// ---- 33 ... 96 rows, dense formats: the eight waves of a workgroup share one staged copy of the states.
+// In the kernel above every wave stages the states of its own units, so a workgroup of 64 columns reads
+// all R x K states: with R = 64 that is four times the packed weights it reads.  Here the waves stand side
+// by side along the columns (32 each, 256 per workgroup), all walk the same units, and each unit's states
+// (16 MT rows x 128 bytes) are moved to LDS once per workgroup, by all 512 threads, a unit ahead of the
+// MFMAs: one barrier per unit.  Thread t stages chunk t % 8 (8 k) of row t / 8 and keeps the running
+// sums of its row over the current quantisation group (sum x, sum off x), which go to LDS with the
+// unit.  K is split across workgroups (blockIdx.z) with the hand-over above, one counter per wave.
+template <int BITS, int MT>
+__global__ __launch_bounds__(512) void wide_rows_kernel(SkinnyArgs a) {
+    using F = SkFmt<BITS>;
+    constexpr int CW = 2, NL = F::LOADS, PF = 4, ROWS = 16 * MT, STRIP = 16 * CW, WSTRIP = 8 * STRIP;
+    constexpr int XBUF = ROWS * SK_PITCH;
+    extern __shared__ __attribute__((aligned(16))) char lds[];
+    typedef typename Words<CW>::type words_t;
+    const int t = threadIdx.x, lane = t & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const int j = lane & 15, h = lane >> 4;
+    const int col0 = blockIdx.x * WSTRIP + wave * STRIP + CW * j;
+    const int units = a.K / 64;
+    const int u0 = blockIdx.z * a.units_per_split, u1 = min(units, u0 + a.units_per_split);
+    const int row0 = blockIdx.y * a.block_rows;
+    const int R = min(a.block_rows, a.R - row0);
+    const int group_lo = u0 / a.group_units;
+    const int groups = (u1 + a.group_units - 1) / a.group_units - group_lo;
+
+    // LDS: two unit buffers, their row sums ([buffer][sum x | sum off x][64]), a flag, the strip's scales and zeros
+    char* const xb = lds;
+    float* const sums = reinterpret_cast<float*>(lds + 2 * XBUF);
+    int* const flag = reinterpret_cast<int*>(lds + 2 * XBUF + 1024);
+    uint32_t* const sz = reinterpret_cast<uint32_t*>(lds + 2 * XBUF + 1024 + 16);
+    auto scan_scales = [&]() -> bool {
+        if (t == 0) *flag = 0;
+        __syncthreads();
+        bool bad = false;
+        const int n = groups * (WSTRIP / 2);
+        for (int i = t; i < n; i += 512) {
+            const int g = i / (WSTRIP / 2), c = i % (WSTRIP / 2);
+            const int64_t at = (int64_t)(group_lo + g) * a.S + blockIdx.x * WSTRIP + 2 * c;
+            const uint32_t two = *reinterpret_cast<const uint32_t*>(a.scales + at);
+            bad |= !(as_h2(two).x >= (h16)0.0f) || !(as_h2(two).y >= (h16)0.0f);
+            sz[i] = two;
+            sz[n + i] = *reinterpret_cast<const uint32_t*>(a.zeros + at);
+        }
+        if (__builtin_amdgcn_ballot_w64(bad) != 0 && lane == 0) *flag = 1;
+        __syncthreads();
+        return *flag != 0;
+    };
+
+    f32x4 acc[CW][MT], y[CW][MT];
+#pragma unroll
+    for (int c = 0; c < CW; ++c)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            acc[c][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+            y[c][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+        }
+
+    // weights of unit u: as in the kernel above (lane group h: chunk h of each of the unit's two blocks)
+    const int wrow = BITS == 4 ? h : (h >> 1);
+    const int wshift = BITS == 4 ? 0 : (BITS == 2 ? 16 * (h & 1) : (h == 0 ? 0 : h == 1 ? 24 : h == 2 ? 16 : 40));
+    const uint32_t* wbase = a.matrix + (int64_t)wrow * a.S + col0;
+    auto load_w = [&](words_t w[NL], int u) {
+        const uint32_t* p = wbase + (int64_t)u * (2 * F::ROWS) * a.S;
+#pragma unroll
+        for (int i = 0; i < NL; ++i) {
+            const int row = BITS == 3 ? 3 * (i >> 1) + (i & 1) : F::ROWS * i;
+            w[i] = __builtin_nontemporal_load(reinterpret_cast<const words_t*>(p + (int64_t)row * a.S));
+        }
+    };
+    auto chunk_bits = [&](const words_t w[NL], int blk, int c) -> uint32_t {
+        if constexpr (BITS == 3)
+            return (uint32_t)((((uint64_t)word_of<CW>(w[2 * blk + 1], c) << 32) | word_of<CW>(w[2 * blk], c)) >> wshift);
+        else
+            return word_of<CW>(w[blk], c) >> wshift;
+    };
+    // states: thread t moves chunk t % 8 of row t / 8
+    const int xrow = t >> 3, xchunk = t & 7;
+    const bool xreal = xrow < R, xstore = xrow < ROWS;
+    const h16* xsrc = a.x + (int64_t)(row0 + min(xrow, R - 1)) * a.K + xchunk * 8;
+    // (every thread loads -- rows beyond R re-read row R - 1 and are zeroed at the staging: a load under a
+    // branch would make the compiler wait for all loads in flight at every use of one)
+    auto load_x = [&](int u) -> u32x4 { return *reinterpret_cast<const u32x4*>(xsrc + u * 64); };
+    float rS = 0.f, rO = 0.f;           // the row's sums over the current group, up to the unit staged last
+    auto stage_x = [&](const u32x4 v, int p, int u) {
+        const uint32_t ONES = 0x3C003C00u;
+        const uint32_t keep = xreal ? 0xFFFFFFFFu : 0u;
+        u32x4 q = u32x4{v[0] & keep, v[1] & keep, v[2] & keep, v[3] & keep};
+        if constexpr (BITS == 4)
+            q = u32x4{__builtin_amdgcn_perm(q[2], q[0], 0x05040100u), __builtin_amdgcn_perm(q[2], q[0], 0x07060302u),
+                      __builtin_amdgcn_perm(q[3], q[1], 0x05040100u), __builtin_amdgcn_perm(q[3], q[1], 0x07060302u)};
+        float sx = 0.f, so = 0.f;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            sx = dot2(q[e], ONES, sx);
+            so = dot2(q[e], F::offs(e), so);
+        }
+        sx += dpp_f32<0xB1>(sx);  so += dpp_f32<0xB1>(so);
+        sx += dpp_f32<0x4E>(sx);  so += dpp_f32<0x4E>(so);
+        sx += dpp_f32<0x141>(sx); so += dpp_f32<0x141>(so);
+        const bool fresh = u == u0 || u % a.group_units == 0;
+        rS = (fresh ? 0.f : rS) + sx;
+        rO = (fresh ? 0.f : rO) + so;
+        if (xstore) {
+            *reinterpret_cast<u32x4*>(xb + p * XBUF + xrow * SK_PITCH + xchunk * 16) = q;
+            if (xchunk == 0) { sums[p * 128 + xrow] = rS; sums[p * 128 + 64 + xrow] = rO; }
+        }
+    };
+
+    words_t w[PF][NL];
+    u32x4 xr[PF];
+    const uint32_t m0 = vgpr_const(BITS == 4 ? 0x000F000Fu : BITS == 2 ? 0x000C0003u : 0x00380007u);
+    const uint32_t g0 = vgpr_const(BITS == 4 ? 0x64006400u : BITS == 2 ? 0x5C006400u : 0x58006400u);
+    const uint32_t m1 = BITS == 4 ? vgpr_const(0x00F000F0u) : 0u, g1 = BITS == 4 ? vgpr_const(0x54005400u) : 0u;
+    h16 sc[CW], ze[CW];
+#pragma unroll
+    for (int c = 0; c < CW; ++c) { sc[c] = (h16)0.f; ze[c] = (h16)0.f; }
+    auto load_sz = [&](int gi) {
+        const h16* ps = reinterpret_cast<const h16*>(sz) + (gi - group_lo) * WSTRIP + wave * STRIP + CW * j;
+        const h16* pz = ps + groups * WSTRIP;
+        const uint32_t s1 = *reinterpret_cast<const uint32_t*>(ps), z1 = *reinterpret_cast<const uint32_t*>(pz);
+        sc[0] = as_h2(s1).x; sc[1] = as_h2(s1).y; ze[0] = as_h2(z1).x; ze[1] = as_h2(z1).y;
+    };
+
+    // set f holds the weights of unit u0 + f; xr[f] the states of unit u0 + 1 + f (unit u0 goes to LDS at once)
+#pragma unroll
+    for (int f = 0; f < PF; ++f) load_w(w[f], min(u0 + f, u1 - 1));
+    {
+        const u32x4 first = load_x(u0);
+#pragma unroll
+        for (int f = 0; f < PF; ++f) xr[f] = load_x(min(u0 + 1 + f, u1 - 1));
+        const bool general = scan_scales();
+        stage_x(first, 0, u0);
+        __syncthreads();
+
+        // p: the LDS buffer that holds unit u; xn: the states of unit u + 1
+        auto step = [&](auto mode, int u, int p, words_t wu[NL], u32x4& xn) {
+            constexpr bool general = decltype(mode)::value;
+            if constexpr (general) {
+                if (u == u0 || u % a.group_units == 0) load_sz(u / a.group_units);
+            }
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                h16x8 xa[MT];
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt)
+                    xa[mt] = *reinterpret_cast<const h16x8*>(xb + p * XBUF + (j + 16 * mt) * SK_PITCH + (i * 4 + h) * 16);
+#pragma unroll
+                for (int c = 0; c < CW; ++c) {
+                    const uint32_t f = chunk_bits(wu, i, c);
+                    const h16x8 wb = general ? exact_operand<BITS>(f, sc[c], ze[c]) : magic_operand<BITS>(f, m0, m1, g0, g1);
+#pragma unroll
+                    for (int mt = 0; mt < MT; ++mt)
+                        acc[c][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[mt], wb, acc[c][mt], 0, 0, 0);
+                }
+            }
+            load_w(wu, min(u + PF, u1 - 1));
+            if (u + 1 < u1) stage_x(xn, p ^ 1, u + 1);
+            xn = load_x(min(u + 1 + PF, u1 - 1));
+            // group complete (or the workgroup's range ends): fold it into y
+            if ((u + 1) % a.group_units == 0 || u + 1 == u1) {
+                if constexpr (!general) load_sz(u / a.group_units);
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) {
+                    const f32x4 s4 = *reinterpret_cast<const f32x4*>(&sums[p * 128 + 16 * mt + 4 * h]);
+                    const f32x4 o4 = *reinterpret_cast<const f32x4*>(&sums[p * 128 + 64 + 16 * mt + 4 * h]);
+#pragma unroll
+                    for (int c = 0; c < CW; ++c) {
+                        const float sf = general ? 1.f : (float)sc[c];
+                        const float z = general ? 0.f : (float)ze[c];
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const float off = general ? 0.f : o4[e] + z * s4[e];
+                            y[c][mt][e] += sf * (acc[c][mt][e] - off);
+                        }
+                        acc[c][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+                    }
+                }
+            }
+            __syncthreads();
+        };
+        auto run = [&](auto mode) {
+            int u = u0;
+            for (; u + PF <= u1; u += PF) {               // (whole rounds without early exits, as above)
+#pragma unroll
+                for (int f = 0; f < PF; ++f) step(mode, u + f, f & 1, w[f], xr[f]);
+            }
+#pragma unroll
+            for (int f = 0; f < PF - 1; ++f) {
+                if (u + f >= u1) break;
+                step(mode, u + f, f & 1, w[f], xr[f]);
+            }
+        };
+        if (general) run(std::integral_constant<bool, true>{});
+        else run(std::integral_constant<bool, false>{});
+    }
+
+    if (gridDim.z > 1) {
+        // hand-over between the workgroups of a strip, wave by wave (see the kernel above)
+        constexpr int NV = CW * MT * 4, THROUGH = 17;
+        const int tile = ((blockIdx.y * gridDim.x + blockIdx.x) << 3) + wave, ks = gridDim.z;
+        char* const slots = reinterpret_cast<char*>(a.part) + (int64_t)tile * ks * (NV * 256);
+        const __amdgpu_buffer_rsrc_t mine = __builtin_amdgcn_make_buffer_rsrc(
+            slots + (int64_t)blockIdx.z * (NV * 256), 0, NV * 256, 0x00020000);
+#pragma unroll
+        for (int c = 0; c < CW; ++c)
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const float v = y[c][mt][e];
+                    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), mine,
+                                                          (((c * MT + mt) * 4 + e) * 64 + lane) * 4, 0, THROUGH);
+                }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_s_waitcnt(0);
+        int arrived = 0;
+        if (lane == 0) arrived = __hip_atomic_fetch_add(a.counters + tile, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        arrived = __builtin_amdgcn_readfirstlane(arrived);
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        if (arrived != ks - 1) return;
+        if (lane == 0) __hip_atomic_store(a.counters + tile, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+        for (int c = 0; c < CW; ++c)
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) y[c][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int sp = 0; sp < ks; ++sp) {
+            const __amdgpu_buffer_rsrc_t theirs = __builtin_amdgcn_make_buffer_rsrc(
+                slots + (int64_t)sp * (NV * 256), 0, NV * 256, 0x00020000);
+#pragma unroll
+            for (int c = 0; c < CW; ++c)
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        y[c][mt][e] += __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                            theirs, (((c * MT + mt) * 4 + e) * 64 + lane) * 4, 0, THROUGH));
+        }
+    }
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int m = mt * 16 + 4 * h + e;
+            if (m < R) {
+                h16* o = a.outs + (int64_t)(row0 + m) * a.S + col0;
+#pragma unroll
+                for (int c = 0; c < CW; ++c) {
+                    float v = y[c][mt][e];
+                    if (a.accumulate) v += (float)o[c];
+                    o[c] = (h16)v;
+                }
+            }
+        }
+}
+
+// Plan of the wide kernel: one or two row blocks of 48 or 64 rows, 256-column strips, K split over about
+// as many workgroups as there are CUs (at least 8 units each, one counter per wave: at most 128 strips
+// and row blocks in all when K is split).
+struct WidePlan { bool use; int mt, row_blocks, block_rows, ksplit, units_per_split; size_t part_bytes; };
+static WidePlan plan_wide(int64_t R, int64_t K, int64_t S, bool sparse) {
+    WidePlan p{false, 0, 0, 0, 1, 0, 0};
+    if (sparse || R < 33 || R > 96 || S % 256 != 0 || K % 64 != 0 || tuning(TUNE_NO_WIDE) != 0) return p;
+    p.row_blocks = R > 64 ? 2 : 1;
+    p.block_rows = (int)(((R + p.row_blocks - 1) / p.row_blocks + 15) / 16 * 16);
+    p.mt = p.block_rows / 16;
+    if (p.mt < 3) { p.mt = 3; p.block_rows = 48; }
+    const int64_t wgs = S / 256 * p.row_blocks, units = K / 64;
+    int64_t ks = std::max<int64_t>(1, std::min<int64_t>(wgs <= 96 ? (256 + wgs / 2) / wgs : 256 / wgs, units / 8));
+    // (two row blocks that cannot be spread over at least three quarters of the CUs: the kernel above is faster)
+    if (p.row_blocks == 2 && wgs * ks < 192) return p;
+    const int64_t forced = tuning(TUNE_MM_SPLIT);
+    if (forced >= 1) ks = std::min<int64_t>(forced, std::max<int64_t>(1, units / 4));
+    if (wgs * 8 > 1024) ks = 1;
+    p.units_per_split = (int)((units + ks - 1) / ks);
+    p.ksplit = (int)((units + p.units_per_split - 1) / p.units_per_split);
+    p.part_bytes = p.ksplit > 1 ? (size_t)wgs * 8 * p.ksplit * (2 * p.mt * 4 * 256) : 0;
+    p.use = true;
+    return p;
+}
+
+template <int BITS>
+static bool launch_wide(SkinnyArgs a, const WidePlan& p, hipStream_t st) {
+    const int upg = a.group_units;
+    int groups = (a.K / 64 + upg - 1) / upg;
+    if (p.ksplit > 1) groups = std::min(groups, (p.units_per_split + upg - 1) / upg + 1);
+    const size_t lds = 2 * (size_t)p.block_rows * SK_PITCH + 1024 + 16 + (size_t)groups * 256 * 4;
+    if (lds > 150 * 1024) return false;
+    a.block_rows = p.block_rows;
+    a.units_per_split = p.units_per_split;
+    const dim3 grid((unsigned)(a.S / 256), (unsigned)p.row_blocks, (unsigned)p.ksplit), block(512);
+    auto go = [&](auto kernel, int slot) {
+        static std::atomic<uint64_t> done[2];
+        int dev = 0;
+        hipGetDevice(&dev);
+        const uint64_t bit = 1ull << (dev & 63);
+        if (!(done[slot].load(std::memory_order_relaxed) & bit)) {
+            hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
+            done[slot].fetch_or(bit, std::memory_order_relaxed);
+        }
+        hipLaunchKernelGGL(kernel, grid, block, lds, st, a);
+    };
+    if (p.mt == 3) go(wide_rows_kernel<BITS, 3>, 0);
+    else go(wide_rows_kernel<BITS, 4>, 1);
+    return true;
+}
+
 template <int BITS, int CW, bool SPARSE>
 static bool launch_skinny(const SkinnyArgs& a, int waves, int ksplit, hipStream_t st) {
     const int strips = a.S / (16 * CW);
@@ -652,7 +960,8 @@ static SkinnySplit plan_skinny_split(int64_t R, int64_t K, int64_t S, bool spars
 
 size_t skinny_workspace_bytes(int64_t R, int64_t K, int64_t S, bool sparse) {
     const SkinnySplit p = plan_skinny_split(R, K, S, sparse);
-    return p.ksplit > 1 ? p.part_bytes : 0;
+    const WidePlan wp = plan_wide(R, K, S, sparse);
+    return std::max<size_t>(p.ksplit > 1 ? p.part_bytes : 0, wp.use ? wp.part_bytes : 0);
 }
 
 // Product of 2 <= R <= 96 rows with a dense or (sparse_mask != nullptr) 16:32 sparse int4 matrix; beyond that
@@ -669,6 +978,21 @@ bool skinny_rows(int bits, h16* outs, const uint32_t* matrix, const h16* x, cons
     const int64_t gu = group_size / 64;
     a.group_units = (int)(gu > 0x7FFFFFF ? 0x7FFFFFF : gu);
     a.accumulate = accumulate ? 1 : 0;
+    a.block_rows = 32;
+    a.part = nullptr;
+    a.counters = nullptr;
+    // 33 rows and more, dense: the kernel whose waves share the staged states
+    {
+        const WidePlan wp = plan_wide(R, K, S, sparse_mask != nullptr);
+        const WorkspaceParts ws = workspace_parts(workspace, workspace_bytes);
+        if (wp.use && (wp.ksplit == 1 || (ws.counters != nullptr && ws.scratch_bytes >= wp.part_bytes))) {
+            a.units_per_wave = 0;
+            a.counters = reinterpret_cast<int*>(ws.counters);
+            a.part = reinterpret_cast<float*>(ws.scratch);
+            const bool ok = bits == 4 ? launch_wide<4>(a, wp, st) : bits == 3 ? launch_wide<3>(a, wp, st) : launch_wide<2>(a, wp, st);
+            if (ok) return true;
+        }
+    }
     // four waves split K when there are 256 workgroups (three of them fit a CU) and K
     // is short (each wave should walk a dozen units or more), eight otherwise
     int cw = unsplit_cw(R, S, sparse_mask != nullptr);

@@ -194,3 +194,41 @@ def test_few_rows_split_k_matvec_entry_accumulates(H):
     p = _problem(4, K=16384, S=256, M=1, B=6, group_size=128, seed=77)
     prior = np.random.default_rng(1).standard_normal((6, 1, 256)).astype(np.float16)
     _check(H, p, "vec", prior=prior)
+
+
+# ---- 33 .. 96 rows, dense formats, S a multiple of 256: the kernel whose eight waves share the staged states
+# (tuning key 8 = 1 switches back to the kernel whose waves stage their own)
+@pytest.mark.parametrize("bits", [4, 3, 2])
+@pytest.mark.parametrize("M,K,S,g", [(33, 1024, 512, 128), (48, 4096, 256, 64), (49, 2048, 768, -1), (64, 8192, 256, 128),
+                                     (65, 1024, 1024, 64), (96, 4096, 512, 128), (80, 320, 256, 64), (40, 64, 256, 64)])
+def test_shared_staging_rows(H, bits, M, K, S, g):
+    capi = H.capi
+    p = _problem(bits, K=K, S=S, M=M, group_size=g, seed=M + K + S)
+    d = H.dev_problem(p)
+    exact, f32 = H.oracles(p)
+    ws = capi.new_matmul_workspace(1, M, K, S, False)
+    runs = []
+    for _ in range(2):
+        o = torch.full((1, M, S), 9.0, dtype=torch.float16, device="cuda")
+        capi.matmul(bits, o, d["matrix"], d["states"], d["scales"], d["zeros"], g, None, ws)
+        torch.cuda.synchronize()
+        runs.append(o.cpu().numpy())
+    H.assert_product_close(runs[0], exact, f32, kind="vec")
+    assert np.array_equal(runs[0], runs[1])
+    capi.tune(8, 1)
+    try:
+        ref = H.run_capi(p, d, "mtx")
+    finally:
+        capi.tune(8, 0)
+    assert O.max_rel_error(ref.astype(np.float64), runs[0]) < H.TOL_EXACT
+
+
+@pytest.mark.parametrize("bits", [4, 3, 2])
+def test_shared_staging_rows_exponent_mode_and_batches(H, bits):
+    p = _problem(bits, K=2048, S=512, M=1, B=50, group_size=128, seed=21)
+    p["scales"][1, 40:48] *= np.float16(-1)
+    p["scales"][9, 300] *= np.float16(-1)
+    prior = np.random.default_rng(5).standard_normal((50, 1, 512)).astype(np.float16)
+    _check(H, p, "vec", prior=prior)                  # the matvec entry adds onto outs
+    q = _problem(bits, K=1024, S=256, M=12, B=4, group_size=64, seed=22)
+    _check(H, q, "mtx")
