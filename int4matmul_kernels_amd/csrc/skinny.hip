@@ -582,9 +582,12 @@ __global__ __launch_bounds__(512) void skinny_kernel(SkinnyArgs a) {
 // all R x K states: with R = 64 that is four times the packed weights it reads.  Here the waves stand side
 // by side along the columns (32 each, 256 per workgroup), all walk the same units, and each unit's states
 // (16 MT rows x 128 bytes) are moved to LDS once per workgroup, by all 512 threads, a unit ahead of the
-// MFMAs: one barrier per unit.  Thread t stages chunk t % 8 (8 k) of row t / 8 and keeps the running
-// sums of its row over the current quantisation group (sum x, sum off x), which go to LDS with the
-// unit.  K is split across workgroups (blockIdx.z) with the hand-over above, one counter per wave.
+// MFMAs: one barrier per unit.  Thread t stages chunk t % 8 (8 k) of row t / 8.  With this many rows the
+// kernel is bound by its vector instructions, and folding scale and zero into the accumulators once per
+// group (3 operations per accumulator element, plus the row sums at the staging) costs more of them than
+// dequantising each weight: the operand is fp16(q s - fp16(z s)), two packed operations per pair of
+// weights on top of the magic-number decode, and the accumulators hold the product itself.
+// K is split across workgroups (blockIdx.z) with the hand-over above, one counter per wave.
 template <int BITS, int MT>
 __global__ __launch_bounds__(512) void wide_rows_kernel(SkinnyArgs a) {
     using F = SkFmt<BITS>;
@@ -603,11 +606,10 @@ __global__ __launch_bounds__(512) void wide_rows_kernel(SkinnyArgs a) {
     const int group_lo = u0 / a.group_units;
     const int groups = (u1 + a.group_units - 1) / a.group_units - group_lo;
 
-    // LDS: two unit buffers, their row sums ([buffer][sum x | sum off x][64]), a flag, the strip's scales and zeros
+    // LDS: two unit buffers, a flag, the strip's scales and zeros
     char* const xb = lds;
-    float* const sums = reinterpret_cast<float*>(lds + 2 * XBUF);
-    int* const flag = reinterpret_cast<int*>(lds + 2 * XBUF + 1024);
-    uint32_t* const sz = reinterpret_cast<uint32_t*>(lds + 2 * XBUF + 1024 + 16);
+    int* const flag = reinterpret_cast<int*>(lds + 2 * XBUF);
+    uint32_t* const sz = reinterpret_cast<uint32_t*>(lds + 2 * XBUF + 16);
     auto scan_scales = [&]() -> bool {
         if (t == 0) *flag = 0;
         __syncthreads();
@@ -626,14 +628,11 @@ __global__ __launch_bounds__(512) void wide_rows_kernel(SkinnyArgs a) {
         return *flag != 0;
     };
 
-    f32x4 acc[CW][MT], y[CW][MT];
+    f32x4 acc[CW][MT];
 #pragma unroll
     for (int c = 0; c < CW; ++c)
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-            acc[c][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
-            y[c][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
-        }
+        for (int mt = 0; mt < MT; ++mt) acc[c][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
     // weights of unit u: as in the kernel above (lane group h: chunk h of each of the unit's two blocks)
     const int wrow = BITS == 4 ? h : (h >> 1);
@@ -655,35 +654,17 @@ __global__ __launch_bounds__(512) void wide_rows_kernel(SkinnyArgs a) {
     };
     // states: thread t moves chunk t % 8 of row t / 8
     const int xrow = t >> 3, xchunk = t & 7;
-    const bool xreal = xrow < R, xstore = xrow < ROWS;
+    const bool xstore = xrow < ROWS;
     const h16* xsrc = a.x + (int64_t)(row0 + min(xrow, R - 1)) * a.K + xchunk * 8;
-    // (every thread loads -- rows beyond R re-read row R - 1 and are zeroed at the staging: a load under a
-    // branch would make the compiler wait for all loads in flight at every use of one)
+    // (every thread loads -- rows beyond R re-read row R - 1, their products are never written: a load
+    // under a branch would make the compiler wait for all loads in flight at every use of one)
     auto load_x = [&](int u) -> u32x4 { return *reinterpret_cast<const u32x4*>(xsrc + u * 64); };
-    float rS = 0.f, rO = 0.f;           // the row's sums over the current group, up to the unit staged last
-    auto stage_x = [&](const u32x4 v, int p, int u) {
-        const uint32_t ONES = 0x3C003C00u;
-        const uint32_t keep = xreal ? 0xFFFFFFFFu : 0u;
-        u32x4 q = u32x4{v[0] & keep, v[1] & keep, v[2] & keep, v[3] & keep};
-        if constexpr (BITS == 4)
-            q = u32x4{__builtin_amdgcn_perm(q[2], q[0], 0x05040100u), __builtin_amdgcn_perm(q[2], q[0], 0x07060302u),
-                      __builtin_amdgcn_perm(q[3], q[1], 0x05040100u), __builtin_amdgcn_perm(q[3], q[1], 0x07060302u)};
-        float sx = 0.f, so = 0.f;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            sx = dot2(q[e], ONES, sx);
-            so = dot2(q[e], F::offs(e), so);
-        }
-        sx += dpp_f32<0xB1>(sx);  so += dpp_f32<0xB1>(so);
-        sx += dpp_f32<0x4E>(sx);  so += dpp_f32<0x4E>(so);
-        sx += dpp_f32<0x141>(sx); so += dpp_f32<0x141>(so);
-        const bool fresh = u == u0 || u % a.group_units == 0;
-        rS = (fresh ? 0.f : rS) + sx;
-        rO = (fresh ? 0.f : rO) + so;
-        if (xstore) {
-            *reinterpret_cast<u32x4*>(xb + p * XBUF + xrow * SK_PITCH + xchunk * 16) = q;
-            if (xchunk == 0) { sums[p * 128 + xrow] = rS; sums[p * 128 + 64 + xrow] = rO; }
-        }
+    auto stage_x = [&](const u32x4 v, int p) {
+        u32x4 q = v;
+        if constexpr (BITS == 4)         // the k order inside the chunk that the operand decode produces
+            q = u32x4{__builtin_amdgcn_perm(v[2], v[0], 0x05040100u), __builtin_amdgcn_perm(v[2], v[0], 0x07060302u),
+                      __builtin_amdgcn_perm(v[3], v[1], 0x05040100u), __builtin_amdgcn_perm(v[3], v[1], 0x07060302u)};
+        if (xstore) *reinterpret_cast<u32x4*>(xb + p * XBUF + xrow * SK_PITCH + xchunk * 16) = q;
     };
 
     words_t w[PF][NL];
@@ -692,13 +673,30 @@ __global__ __launch_bounds__(512) void wide_rows_kernel(SkinnyArgs a) {
     const uint32_t g0 = vgpr_const(BITS == 4 ? 0x64006400u : BITS == 2 ? 0x5C006400u : 0x58006400u);
     const uint32_t m1 = BITS == 4 ? vgpr_const(0x00F000F0u) : 0u, g1 = BITS == 4 ? vgpr_const(0x54005400u) : 0u;
     h16 sc[CW], ze[CW];
+    h16x2 s2[CW], c2[CW];               // {s, s} and {-fp16(z s), -fp16(z s)} of the lane's columns
 #pragma unroll
-    for (int c = 0; c < CW; ++c) { sc[c] = (h16)0.f; ze[c] = (h16)0.f; }
+    for (int c = 0; c < CW; ++c) { sc[c] = (h16)0.f; ze[c] = (h16)0.f; s2[c] = h16x2{(h16)0.f, (h16)0.f}; c2[c] = s2[c]; }
     auto load_sz = [&](int gi) {
         const h16* ps = reinterpret_cast<const h16*>(sz) + (gi - group_lo) * WSTRIP + wave * STRIP + CW * j;
         const h16* pz = ps + groups * WSTRIP;
         const uint32_t s1 = *reinterpret_cast<const uint32_t*>(ps), z1 = *reinterpret_cast<const uint32_t*>(pz);
         sc[0] = as_h2(s1).x; sc[1] = as_h2(s1).y; ze[0] = as_h2(z1).x; ze[1] = as_h2(z1).y;
+#pragma unroll
+        for (int c = 0; c < CW; ++c) {
+            const h16 zs = -(ze[c] * sc[c]);
+            s2[c] = h16x2{sc[c], sc[c]};
+            c2[c] = h16x2{zs, zs};
+        }
+    };
+    // the chunk's magic numbers minus their offsets are the codes, exactly; then one packed fma each
+    auto scaled_operand = [&](uint32_t f, int c) -> h16x8 {
+        u32x4 r = bitcast<u32x4>(magic_operand<BITS>(f, m0, m1, g0, g1));
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const h16x2 q = as_h2(r[e]) - as_h2(F::offs(e));
+            r[e] = bitcast<uint32_t>(__builtin_elementwise_fma(q, s2[c], c2[c]));
+        }
+        return bitcast<h16x8>(r);
     };
 
     // set f holds the weights of unit u0 + f; xr[f] the states of unit u0 + 1 + f (unit u0 goes to LDS at once)
@@ -709,15 +707,13 @@ __global__ __launch_bounds__(512) void wide_rows_kernel(SkinnyArgs a) {
 #pragma unroll
         for (int f = 0; f < PF; ++f) xr[f] = load_x(min(u0 + 1 + f, u1 - 1));
         const bool general = scan_scales();
-        stage_x(first, 0, u0);
+        stage_x(first, 0);
         __syncthreads();
 
         // p: the LDS buffer that holds unit u; xn: the states of unit u + 1
         auto step = [&](auto mode, int u, int p, words_t wu[NL], u32x4& xn) {
             constexpr bool general = decltype(mode)::value;
-            if constexpr (general) {
-                if (u == u0 || u % a.group_units == 0) load_sz(u / a.group_units);
-            }
+            if (u == u0 || u % a.group_units == 0) load_sz(u / a.group_units);
 #pragma unroll
             for (int i = 0; i < 2; ++i) {
                 h16x8 xa[MT];
@@ -727,35 +723,15 @@ __global__ __launch_bounds__(512) void wide_rows_kernel(SkinnyArgs a) {
 #pragma unroll
                 for (int c = 0; c < CW; ++c) {
                     const uint32_t f = chunk_bits(wu, i, c);
-                    const h16x8 wb = general ? exact_operand<BITS>(f, sc[c], ze[c]) : magic_operand<BITS>(f, m0, m1, g0, g1);
+                    const h16x8 wb = general ? exact_operand<BITS>(f, sc[c], ze[c]) : scaled_operand(f, c);
 #pragma unroll
                     for (int mt = 0; mt < MT; ++mt)
                         acc[c][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[mt], wb, acc[c][mt], 0, 0, 0);
                 }
             }
             load_w(wu, min(u + PF, u1 - 1));
-            if (u + 1 < u1) stage_x(xn, p ^ 1, u + 1);
+            if (u + 1 < u1) stage_x(xn, p ^ 1);
             xn = load_x(min(u + 1 + PF, u1 - 1));
-            // group complete (or the workgroup's range ends): fold it into y
-            if ((u + 1) % a.group_units == 0 || u + 1 == u1) {
-                if constexpr (!general) load_sz(u / a.group_units);
-#pragma unroll
-                for (int mt = 0; mt < MT; ++mt) {
-                    const f32x4 s4 = *reinterpret_cast<const f32x4*>(&sums[p * 128 + 16 * mt + 4 * h]);
-                    const f32x4 o4 = *reinterpret_cast<const f32x4*>(&sums[p * 128 + 64 + 16 * mt + 4 * h]);
-#pragma unroll
-                    for (int c = 0; c < CW; ++c) {
-                        const float sf = general ? 1.f : (float)sc[c];
-                        const float z = general ? 0.f : (float)ze[c];
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) {
-                            const float off = general ? 0.f : o4[e] + z * s4[e];
-                            y[c][mt][e] += sf * (acc[c][mt][e] - off);
-                        }
-                        acc[c][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
-                    }
-                }
-            }
             __syncthreads();
         };
         auto run = [&](auto mode) {
@@ -787,7 +763,7 @@ __global__ __launch_bounds__(512) void wide_rows_kernel(SkinnyArgs a) {
             for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    const float v = y[c][mt][e];
+                    const float v = acc[c][mt][e];
                     __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), mine,
                                                           (((c * MT + mt) * 4 + e) * 64 + lane) * 4, 0, THROUGH);
                 }
@@ -802,7 +778,7 @@ __global__ __launch_bounds__(512) void wide_rows_kernel(SkinnyArgs a) {
 #pragma unroll
         for (int c = 0; c < CW; ++c)
 #pragma unroll
-            for (int mt = 0; mt < MT; ++mt) y[c][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+            for (int mt = 0; mt < MT; ++mt) acc[c][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
         for (int sp = 0; sp < ks; ++sp) {
             const __amdgpu_buffer_rsrc_t theirs = __builtin_amdgcn_make_buffer_rsrc(
                 slots + (int64_t)sp * (NV * 256), 0, NV * 256, 0x00020000);
@@ -812,7 +788,7 @@ __global__ __launch_bounds__(512) void wide_rows_kernel(SkinnyArgs a) {
                 for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
                     for (int e = 0; e < 4; ++e)
-                        y[c][mt][e] += __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                        acc[c][mt][e] += __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
                             theirs, (((c * MT + mt) * 4 + e) * 64 + lane) * 4, 0, THROUGH));
         }
     }
@@ -825,7 +801,7 @@ __global__ __launch_bounds__(512) void wide_rows_kernel(SkinnyArgs a) {
                 h16* o = a.outs + (int64_t)(row0 + m) * a.S + col0;
 #pragma unroll
                 for (int c = 0; c < CW; ++c) {
-                    float v = y[c][mt][e];
+                    float v = acc[c][mt][e];
                     if (a.accumulate) v += (float)o[c];
                     o[c] = (h16)v;
                 }
@@ -839,11 +815,12 @@ __global__ __launch_bounds__(512) void wide_rows_kernel(SkinnyArgs a) {
 struct WidePlan { bool use; int mt, row_blocks, block_rows, ksplit, units_per_split; size_t part_bytes; };
 static WidePlan plan_wide(int64_t R, int64_t K, int64_t S, bool sparse) {
     WidePlan p{false, 0, 0, 0, 1, 0, 0};
-    if (sparse || R < 33 || R > 96 || S % 256 != 0 || K % 64 != 0 || tuning(TUNE_NO_WIDE) != 0) return p;
+    // (knob: 1 = never, n >= 2 = from n rows on whatever the shape)
+    const int64_t knob = tuning(TUNE_NO_WIDE), min_rows = knob >= 2 ? knob : 17;
+    if (sparse || R < min_rows || R > 96 || S % 256 != 0 || K % 64 != 0 || knob == 1) return p;
     p.row_blocks = R > 64 ? 2 : 1;
     p.block_rows = (int)(((R + p.row_blocks - 1) / p.row_blocks + 15) / 16 * 16);
     p.mt = p.block_rows / 16;
-    if (p.mt < 3) { p.mt = 3; p.block_rows = 48; }
     const int64_t wgs = S / 256 * p.row_blocks, units = K / 64;
     int64_t ks = std::max<int64_t>(1, std::min<int64_t>(wgs <= 96 ? (256 + wgs / 2) / wgs : 256 / wgs, units / 8));
     // (two row blocks that cannot be spread over at least three quarters of the CUs: the kernel above is faster)
@@ -853,6 +830,12 @@ static WidePlan plan_wide(int64_t R, int64_t K, int64_t S, bool sparse) {
     if (wgs * 8 > 1024) ks = 1;
     p.units_per_split = (int)((units + ks - 1) / ks);
     p.ksplit = (int)((units + p.units_per_split - 1) / p.units_per_split);
+    // measured against the kernel above (K = 2048 ... 20480, S = 1024 ... 28672): with 17 ... 32 rows it
+    // needs wide matrices and long shares of K, with 33 ... 64 rows matrices of 32 M weights and more
+    if (knob < 2 && forced < 1) {
+        if (R <= 32 && (wgs < 32 || p.units_per_split < 16)) return p;
+        if (R > 32 && R <= 64 && K * S < (1ll << 25)) return p;
+    }
     p.part_bytes = p.ksplit > 1 ? (size_t)wgs * 8 * p.ksplit * (2 * p.mt * 4 * 256) : 0;
     p.use = true;
     return p;
@@ -869,7 +852,7 @@ static bool launch_wide(SkinnyArgs a, const WidePlan& p, hipStream_t st) {
     a.units_per_split = p.units_per_split;
     const dim3 grid((unsigned)(a.S / 256), (unsigned)p.row_blocks, (unsigned)p.ksplit), block(512);
     auto go = [&](auto kernel, int slot) {
-        static std::atomic<uint64_t> done[2];
+        static std::atomic<uint64_t> done[4];
         int dev = 0;
         hipGetDevice(&dev);
         const uint64_t bit = 1ull << (dev & 63);
@@ -879,8 +862,10 @@ static bool launch_wide(SkinnyArgs a, const WidePlan& p, hipStream_t st) {
         }
         hipLaunchKernelGGL(kernel, grid, block, lds, st, a);
     };
-    if (p.mt == 3) go(wide_rows_kernel<BITS, 3>, 0);
-    else go(wide_rows_kernel<BITS, 4>, 1);
+    if (p.mt == 1) go(wide_rows_kernel<BITS, 1>, 0);
+    else if (p.mt == 2) go(wide_rows_kernel<BITS, 2>, 1);
+    else if (p.mt == 3) go(wide_rows_kernel<BITS, 3>, 2);
+    else go(wide_rows_kernel<BITS, 4>, 3);
     return true;
 }
 

@@ -200,19 +200,24 @@ def test_few_rows_split_k_matvec_entry_accumulates(H):
 # (tuning key 8 = 1 switches back to the kernel whose waves stage their own)
 @pytest.mark.parametrize("bits", [4, 3, 2])
 @pytest.mark.parametrize("M,K,S,g", [(33, 1024, 512, 128), (48, 4096, 256, 64), (49, 2048, 768, -1), (64, 8192, 256, 128),
-                                     (65, 1024, 1024, 64), (96, 4096, 512, 128), (80, 320, 256, 64), (40, 64, 256, 64)])
+                                     (65, 1024, 1024, 64), (96, 4096, 512, 128), (80, 320, 256, 64), (40, 64, 256, 64),
+                                     (2, 2048, 256, 128), (16, 1024, 512, 64), (17, 4096, 256, 128), (32, 2048, 512, -1)])
 def test_shared_staging_rows(H, bits, M, K, S, g):
     capi = H.capi
     p = _problem(bits, K=K, S=S, M=M, group_size=g, seed=M + K + S)
     d = H.dev_problem(p)
     exact, f32 = H.oracles(p)
-    ws = capi.new_matmul_workspace(1, M, K, S, False)
     runs = []
-    for _ in range(2):
-        o = torch.full((1, M, S), 9.0, dtype=torch.float16, device="cuda")
-        capi.matmul(bits, o, d["matrix"], d["states"], d["scales"], d["zeros"], g, None, ws)
-        torch.cuda.synchronize()
-        runs.append(o.cpu().numpy())
+    capi.tune(8, 2)                          # whatever the shape (by default: large matrices only)
+    try:
+        ws = capi.new_matmul_workspace(1, M, K, S, False)
+        for _ in range(2):
+            o = torch.full((1, M, S), 9.0, dtype=torch.float16, device="cuda")
+            capi.matmul(bits, o, d["matrix"], d["states"], d["scales"], d["zeros"], g, None, ws)
+            torch.cuda.synchronize()
+            runs.append(o.cpu().numpy())
+    finally:
+        capi.tune(8, 0)
     H.assert_product_close(runs[0], exact, f32, kind="vec")
     assert np.array_equal(runs[0], runs[1])
     capi.tune(8, 1)
@@ -225,6 +230,14 @@ def test_shared_staging_rows(H, bits, M, K, S, g):
 
 @pytest.mark.parametrize("bits", [4, 3, 2])
 def test_shared_staging_rows_exponent_mode_and_batches(H, bits):
+    H.capi.tune(8, 2)
+    try:
+        _shared_staging_exponent_and_batches(H, bits)
+    finally:
+        H.capi.tune(8, 0)
+
+
+def _shared_staging_exponent_and_batches(H, bits):
     p = _problem(bits, K=2048, S=512, M=1, B=50, group_size=128, seed=21)
     p["scales"][1, 40:48] *= np.float16(-1)
     p["scales"][9, 300] *= np.float16(-1)
@@ -232,3 +245,10 @@ def test_shared_staging_rows_exponent_mode_and_batches(H, bits):
     _check(H, p, "vec", prior=prior)                  # the matvec entry adds onto outs
     q = _problem(bits, K=1024, S=256, M=12, B=4, group_size=64, seed=22)
     _check(H, q, "mtx")
+
+
+@pytest.mark.parametrize("M", [17, 32, 40, 64, 96])
+def test_shared_staging_rows_default_rule_large_matrix(H, M):
+    """K=4096, S=8192 (32 M weights): every row count from 17 on takes the shared-staging kernel by default"""
+    p = _problem(4, K=4096, S=8192, M=M, group_size=128, seed=M)
+    _check(H, p, "mtx")
