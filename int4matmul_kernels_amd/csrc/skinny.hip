@@ -809,7 +809,7 @@ __global__ __launch_bounds__(512) void wide_rows_kernel(SkinnyArgs a) {
         }
 }
 
-// Plan of the wide kernel: one or two row blocks of 48 or 64 rows, 256-column strips, K split over about
+// Plan of the wide kernel: one or two row blocks of 16 ... 64 rows, 256-column strips, K split over about
 // as many workgroups as there are CUs (at least 8 units each, one counter per wave: at most 128 strips
 // and row blocks in all when K is split).
 struct WidePlan { bool use; int mt, row_blocks, block_rows, ksplit, units_per_split; size_t part_bytes; };
@@ -822,9 +822,11 @@ static WidePlan plan_wide(int64_t R, int64_t K, int64_t S, bool sparse) {
     p.block_rows = (int)(((R + p.row_blocks - 1) / p.row_blocks + 15) / 16 * 16);
     p.mt = p.block_rows / 16;
     const int64_t wgs = S / 256 * p.row_blocks, units = K / 64;
-    int64_t ks = std::max<int64_t>(1, std::min<int64_t>(wgs <= 96 ? (256 + wgs / 2) / wgs : 256 / wgs, units / 8));
-    // (two row blocks that cannot be spread over at least three quarters of the CUs: the kernel above is faster)
-    if (p.row_blocks == 2 && wgs * ks < 192) return p;
+    // (one workgroup per CU: as many splits as keep the grid within one round of 256 -- a grid a little larger
+    // than that runs a second round -- and four when even the unsplit grid leaves a third of the CUs idle)
+    int64_t ks = 256 / wgs;
+    if (ks <= 1 && wgs > 128 && wgs < 256) ks = 4;
+    ks = std::max<int64_t>(1, std::min<int64_t>(ks, units / 8));
     const int64_t forced = tuning(TUNE_MM_SPLIT);
     if (forced >= 1) ks = std::min<int64_t>(forced, std::max<int64_t>(1, units / 4));
     if (wgs * 8 > 1024) ks = 1;
