@@ -1039,7 +1039,7 @@ extern "C" int int4mm_matmul(int bits, void* outs, const void* matrix, const voi
 
     hipStream_t st = (hipStream_t)stream;
     // 2 .. 96 rows in all (batches are contiguous, so they flatten): the HBM-bound few-row kernel
-    if (B * M >= 2 && B * M <= 96 && !tuning(TUNE_NO_SKINNY) &&
+    if (B * M >= 2 && B * M <= SK_WIDE_MAX_ROWS && !tuning(TUNE_NO_SKINNY) &&
         skinny_rows(bits, (h16*)outs, (const uint32_t*)matrix, (const h16*)multiplier, (const h16*)scales,
                     (const h16*)zeros, B * M, K, S, g, false, st, (const uint32_t*)sparse_mask, workspace, workspace_bytes))
         return check_launch("matmul");
@@ -1076,9 +1076,11 @@ extern "C" size_t int4mm_matmul_workspace_bytes(const int4mm_shape* shape, int s
     const int64_t B = shape->batch, M = shape->seq_len, K = shape->in_size, S = shape->out_size;
     size_t need = int4mm_workspace_bytes(S);
     if (B <= 0 || M <= 0 || K < 64 || S < 128) return need;
-    if (B * M <= 96) return need + 2 * round_to_page(skinny_workspace_bytes(B * M, K, S, sparse != 0));
+    const size_t few_rows = B * M <= SK_WIDE_MAX_ROWS ? skinny_workspace_bytes(B * M, K, S, sparse != 0) : 0;
+    if (B * M <= 96) return need + 2 * round_to_page(few_rows);
     const SplitPlan sp = plan_split(sparse != 0, B, M, K, S);
-    if (sp.ksplit > 1) need += 2 * round_to_page((size_t)(sp.tiles * sp.ksplit * sp.tile_bytes));
+    if (sp.ksplit > 1 || few_rows > 0)
+        need += 2 * round_to_page(std::max(few_rows, sp.ksplit > 1 ? (size_t)(sp.tiles * sp.ksplit * sp.tile_bytes) : 0));
     const TailPlan tp = plan_tail(B, M, K, S);
     if (sp.ksplit == 1 && tp.ksplit > 1) need += 2 * round_to_page((size_t)(tp.tiles * tp.ksplit * (256 * 256 * 4)));
     return need;

@@ -721,7 +721,7 @@ extern "C" int int4mm_matvec(int bits, void* outs, const void* matrix, const voi
     const int64_t g = shape->group_size < 0 ? ONE_GROUP : shape->group_size;
 
     // several batch elements of one row each: one pass over the weights for all of them
-    if (B >= 2 && B <= 96 && !tuning(TUNE_NO_SKINNY) &&
+    if (B >= 2 && B <= SK_WIDE_MAX_ROWS && !tuning(TUNE_NO_SKINNY) &&
         skinny_rows(bits, (h16*)outs, (const uint32_t*)matrix, (const h16*)multiplier, (const h16*)scales,
                     (const h16*)zeros, B, K, S, g, true, (hipStream_t)stream, (const uint32_t*)sparse_mask, workspace, workspace_bytes))
         return check_launch("matvec");

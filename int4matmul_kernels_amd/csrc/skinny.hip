@@ -585,8 +585,8 @@ __global__ __launch_bounds__(512) void skinny_kernel(SkinnyArgs a) {
 // MFMAs: one barrier per unit.  Thread t stages chunk t % 8 (8 k) of row t / 8.  With this many rows the
 // kernel is bound by its vector instructions, and folding scale and zero into the accumulators once per
 // group (3 operations per accumulator element, plus the row sums at the staging) costs more of them than
-// dequantising each weight: the operand is fp16(q s - fp16(z s)), two packed operations per pair of
-// weights on top of the magic-number decode, and the accumulators hold the product itself.
+// dequantising each weight: the operand is the reference's fp16(fp16(q - z) s), three packed operations
+// per pair of weights on top of the magic-number decode, and the accumulators hold the product itself.
 // K is split across workgroups (blockIdx.z) with the hand-over above, one counter per wave.
 template <int BITS, int MT>
 __global__ __launch_bounds__(512) void wide_rows_kernel(SkinnyArgs a) {
@@ -673,7 +673,7 @@ __global__ __launch_bounds__(512) void wide_rows_kernel(SkinnyArgs a) {
     const uint32_t g0 = vgpr_const(BITS == 4 ? 0x64006400u : BITS == 2 ? 0x5C006400u : 0x58006400u);
     const uint32_t m1 = BITS == 4 ? vgpr_const(0x00F000F0u) : 0u, g1 = BITS == 4 ? vgpr_const(0x54005400u) : 0u;
     h16 sc[CW], ze[CW];
-    h16x2 s2[CW], c2[CW];               // {s, s} and {-fp16(z s), -fp16(z s)} of the lane's columns
+    h16x2 s2[CW], c2[CW];               // {s, s} and {z, z} of the lane's columns
 #pragma unroll
     for (int c = 0; c < CW; ++c) { sc[c] = (h16)0.f; ze[c] = (h16)0.f; s2[c] = h16x2{(h16)0.f, (h16)0.f}; c2[c] = s2[c]; }
     auto load_sz = [&](int gi) {
@@ -683,18 +683,18 @@ __global__ __launch_bounds__(512) void wide_rows_kernel(SkinnyArgs a) {
         sc[0] = as_h2(s1).x; sc[1] = as_h2(s1).y; ze[0] = as_h2(z1).x; ze[1] = as_h2(z1).y;
 #pragma unroll
         for (int c = 0; c < CW; ++c) {
-            const h16 zs = -(ze[c] * sc[c]);
             s2[c] = h16x2{sc[c], sc[c]};
-            c2[c] = h16x2{zs, zs};
+            c2[c] = h16x2{ze[c], ze[c]};
         }
     };
-    // the chunk's magic numbers minus their offsets are the codes, exactly; then one packed fma each
+    // the chunk's magic numbers minus their offsets are the codes, exactly; then the reference's own
+    // two roundings: fp16(fp16(q - z) s) (matmul.cuh:115-125)
     auto scaled_operand = [&](uint32_t f, int c) -> h16x8 {
         u32x4 r = bitcast<u32x4>(magic_operand<BITS>(f, m0, m1, g0, g1));
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
             const h16x2 q = as_h2(r[e]) - as_h2(F::offs(e));
-            r[e] = bitcast<uint32_t>(__builtin_elementwise_fma(q, s2[c], c2[c]));
+            r[e] = bitcast<uint32_t>((q - c2[c]) * s2[c]);
         }
         return bitcast<h16x8>(r);
     };
@@ -751,12 +751,13 @@ __global__ __launch_bounds__(512) void wide_rows_kernel(SkinnyArgs a) {
     }
 
     if (gridDim.z > 1) {
-        // hand-over between the workgroups of a strip, wave by wave (see the kernel above)
+        // hand-over between the workgroups of a strip (see the kernel above): every wave stores its part of
+        // the workgroup's partial tile, one counter per strip and row block
         constexpr int NV = CW * MT * 4, THROUGH = 17;
-        const int tile = ((blockIdx.y * gridDim.x + blockIdx.x) << 3) + wave, ks = gridDim.z;
-        char* const slots = reinterpret_cast<char*>(a.part) + (int64_t)tile * ks * (NV * 256);
+        const int tile = blockIdx.y * gridDim.x + blockIdx.x, ks = gridDim.z;
+        char* const slots = reinterpret_cast<char*>(a.part) + ((int64_t)(tile * ks) * 8 + wave) * (NV * 256);
         const __amdgpu_buffer_rsrc_t mine = __builtin_amdgcn_make_buffer_rsrc(
-            slots + (int64_t)blockIdx.z * (NV * 256), 0, NV * 256, 0x00020000);
+            slots + (int64_t)blockIdx.z * (8 * NV * 256), 0, NV * 256, 0x00020000);
 #pragma unroll
         for (int c = 0; c < CW; ++c)
 #pragma unroll
@@ -767,21 +768,19 @@ __global__ __launch_bounds__(512) void wide_rows_kernel(SkinnyArgs a) {
                     __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), mine,
                                                           (((c * MT + mt) * 4 + e) * 64 + lane) * 4, 0, THROUGH);
                 }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_s_waitcnt(0);
-        int arrived = 0;
-        if (lane == 0) arrived = __hip_atomic_fetch_add(a.counters + tile, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        arrived = __builtin_amdgcn_readfirstlane(arrived);
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-        if (arrived != ks - 1) return;
-        if (lane == 0) __hip_atomic_store(a.counters + tile, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __builtin_amdgcn_s_waitcnt(0);                 // every store of this thread has been acknowledged
+        __syncthreads();
+        if (t == 0) *flag = __hip_atomic_fetch_add(a.counters + tile, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        if (*flag != ks - 1) return;
+        if (t == 0) __hip_atomic_store(a.counters + tile, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 #pragma unroll
         for (int c = 0; c < CW; ++c)
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) acc[c][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
         for (int sp = 0; sp < ks; ++sp) {
             const __amdgpu_buffer_rsrc_t theirs = __builtin_amdgcn_make_buffer_rsrc(
-                slots + (int64_t)sp * (NV * 256), 0, NV * 256, 0x00020000);
+                slots + (int64_t)sp * (8 * NV * 256), 0, NV * 256, 0x00020000);
 #pragma unroll
             for (int c = 0; c < CW; ++c)
 #pragma unroll
@@ -809,16 +808,15 @@ __global__ __launch_bounds__(512) void wide_rows_kernel(SkinnyArgs a) {
         }
 }
 
-// Plan of the wide kernel: one or two row blocks of 16 ... 64 rows, 256-column strips, K split over about
-// as many workgroups as there are CUs (at least 8 units each, one counter per wave: at most 128 strips
-// and row blocks in all when K is split).
+// Plan of the wide kernel: row blocks of 16 ... 64 rows, 256-column strips, K split over about as many
+// workgroups as there are CUs (at least 8 units each; one counter per strip and row block: at most 1024).
 struct WidePlan { bool use; int mt, row_blocks, block_rows, ksplit, units_per_split; size_t part_bytes; };
 static WidePlan plan_wide(int64_t R, int64_t K, int64_t S, bool sparse) {
     WidePlan p{false, 0, 0, 0, 1, 0, 0};
     // (knob: 1 = never, n >= 2 = from n rows on whatever the shape)
     const int64_t knob = tuning(TUNE_NO_WIDE), min_rows = knob >= 2 ? knob : 17;
-    if (sparse || R < min_rows || R > 96 || S % 256 != 0 || K % 64 != 0 || knob == 1) return p;
-    p.row_blocks = R > 64 ? 2 : 1;
+    if (sparse || R < min_rows || R > SK_WIDE_MAX_ROWS || S % 256 != 0 || K % 64 != 0 || knob == 1) return p;
+    p.row_blocks = (int)((R + 63) / 64);
     p.block_rows = (int)(((R + p.row_blocks - 1) / p.row_blocks + 15) / 16 * 16);
     p.mt = p.block_rows / 16;
     const int64_t wgs = S / 256 * p.row_blocks, units = K / 64;
@@ -829,14 +827,16 @@ static WidePlan plan_wide(int64_t R, int64_t K, int64_t S, bool sparse) {
     ks = std::max<int64_t>(1, std::min<int64_t>(ks, units / 8));
     const int64_t forced = tuning(TUNE_MM_SPLIT);
     if (forced >= 1) ks = std::min<int64_t>(forced, std::max<int64_t>(1, units / 4));
-    if (wgs * 8 > 1024) ks = 1;
+    if (wgs > 1024) ks = 1;
     p.units_per_split = (int)((units + ks - 1) / ks);
     p.ksplit = (int)((units + p.units_per_split - 1) / p.units_per_split);
     // measured against the kernel above (K = 2048 ... 20480, S = 1024 ... 28672): with 17 ... 32 rows it
     // needs wide matrices and long shares of K, with 33 ... 64 rows matrices of 32 M weights and more
+    // and from 129 rows on the tile kernels win on wide outputs
     if (knob < 2 && forced < 1) {
         if (R <= 32 && (wgs < 32 || p.units_per_split < 16)) return p;
         if (R > 32 && R <= 64 && K * S < (1ll << 25)) return p;
+        if (R > 128 && S > 8192) return p;
     }
     p.part_bytes = p.ksplit > 1 ? (size_t)wgs * 8 * p.ksplit * (2 * p.mt * 4 * 256) : 0;
     p.use = true;
@@ -957,7 +957,7 @@ size_t skinny_workspace_bytes(int64_t R, int64_t K, int64_t S, bool sparse) {
 bool skinny_rows(int bits, h16* outs, const uint32_t* matrix, const h16* x, const h16* scales, const h16* zeros,
                  int64_t R, int64_t K, int64_t S, int64_t group_size, bool accumulate, hipStream_t st,
                  const uint32_t* sparse_mask, void* workspace, size_t workspace_bytes) {
-    if (R < 2 || R > 96 || S % 16 != 0 || K % 64 != 0 || K > (1 << 30) || S > (1 << 28)) return false;
+    if (R < 2 || R > SK_WIDE_MAX_ROWS || S % 16 != 0 || K % 64 != 0 || K > (1 << 30) || S > (1 << 28)) return false;
     if (sparse_mask && bits != 4) return false;
     SkinnyArgs a;
     a.outs = outs; a.matrix = matrix; a.mask = sparse_mask; a.x = x; a.scales = scales; a.zeros = zeros;
@@ -980,6 +980,7 @@ bool skinny_rows(int bits, h16* outs, const uint32_t* matrix, const h16* x, cons
             if (ok) return true;
         }
     }
+    if (R > 96) return false;
     // four waves split K when there are 256 workgroups (three of them fit a CU) and K
     // is short (each wave should walk a dozen units or more), eight otherwise
     int cw = unsplit_cw(R, S, sparse_mask != nullptr);

@@ -252,3 +252,22 @@ def test_shared_staging_rows_default_rule_large_matrix(H, M):
     """K=4096, S=8192 (32 M weights): every row count from 17 on takes the shared-staging kernel by default"""
     p = _problem(4, K=4096, S=8192, M=M, group_size=128, seed=M)
     _check(H, p, "mtx")
+
+
+@pytest.mark.parametrize("bits", [4, 3, 2])
+@pytest.mark.parametrize("M,K,S,g", [(97, 1024, 512, 128), (128, 4096, 256, 64), (130, 2048, 768, -1), (200, 1024, 1024, 64),
+                                     (256, 2048, 512, 128), (129, 320, 256, 64)])
+def test_shared_staging_up_to_256_rows(H, bits, M, K, S, g):
+    """97 ... 256 rows (up to four row blocks of 64): the weights are dequantised with the reference's two
+    roundings, so the matmul tolerance against the product on fp16 weights holds"""
+    p = _problem(bits, K=K, S=S, M=M, group_size=g, seed=M + K + S)
+    d = H.dev_problem(p)
+    exact, f32 = H.oracles(p)
+    got = H.run_capi(p, d, "mtx", outs_init=np.full((1, M, S), 2.0, np.float16))
+    H.assert_product_close(got, exact, f32, kind="mtx")
+    H.capi.tune(8, 1)
+    try:
+        ref = H.run_capi(p, d, "mtx")
+    finally:
+        H.capi.tune(8, 0)
+    assert O.max_rel_error(ref.astype(np.float64), got) < H.TOL_EXACT_MTX

@@ -16,7 +16,9 @@ from oracle import oracle as O  # noqa: E402
 @pytest.fixture(scope="module")
 def H():
     from tests import helpers
-    return helpers
+    helpers.capi.tune(8, 1)          # (up to 256 rows would otherwise take the few-row path: not the subject here)
+    yield helpers
+    helpers.capi.tune(8, 0)
 
 
 def _problem(bits, sparse, **kw):
