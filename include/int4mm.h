@@ -71,8 +71,11 @@ INT4MM_API int int4mm_abi_version(void);
  * group, 2 = matvec lane groups per wave (1, 2, 4), 3 = matmul kernel variant
  * (5 / 6 = pipelined 256x128 / 256x256 tiles, 9 = 256x256 without the two-phase
  * order), 4 = matvec: 1 disables prefetch,
- * 5 = 1 disables the few-row (2..96 rows) kernel, 6 = matmul split-K factor
- * (1 = never split, 2..8 = that factor where the shape allows a split at all). */
+ * 5 = 1 disables the few-row (2..256 rows) kernels, 6 = split-K factor of the
+ * matmul and few-row kernels (1 = never split, 2..8 = that factor where the
+ * shape allows a split at all), 7 = 1: the tiles of a matmul's last, partly
+ * filled round are not split, 8 = the few-row kernel whose waves share the
+ * staged states: 1 = never, n >= 2 = from n rows on whatever the shape. */
 INT4MM_API int int4mm_tune(int key, int64_t value);
 
 /* Shape of one product.  matrix_rows = R, n_groups = G (rows of scales/zeros).
@@ -106,7 +109,7 @@ INT4MM_API int int4mm_workspace_init(void* workspace, size_t workspace_bytes, vo
 /* Bytes of workspace with which int4mm_matmul may split the K dimension of `shape`
  * over several workgroups per output tile (shapes with so few tiles that most of
  * the GPU would idle, or whose last round of tiles would leave half of it idle; `sparse` != 0 for the 16:32 format) -- also int4mm_matvec
- * with 2 .. 96 batch entries, which takes the few-row kernel; never less than
+ * with 2 .. 256 batch entries, which takes the few-row kernels; never less than
  * int4mm_workspace_bytes(shape->out_size).  A smaller workspace is not an error:
  * the product then runs unsplit.  Same zero-fill rule as above.  No counterpart in
  * the reference, whose matmul (matmul_kernel.cu:375-459) uses no scratch. */

@@ -1,5 +1,5 @@
-"""The few-row kernel (2 .. 96 rows of states in all; dense formats and 16:32
-sparse int4): every packed word is read once for all rows.  It serves `quant_matmul` with small M (any
+"""The few-row kernels (2 .. 96 rows of states in all, dense formats on suitable shapes up to 256; dense
+formats and 16:32 sparse int4): every packed word is read once for all rows.  It serves `quant_matmul` with small M (any
 batch layout that flattens to <= 32 rows) and the matvec entry with B > 1.
 Its numerics are the matvec's (exact sum of x (q - z) s, no per-weight fp16
 rounding), so the matvec tolerance applies; it is also checked against the
