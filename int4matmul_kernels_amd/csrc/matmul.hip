@@ -970,11 +970,15 @@ static void launch(MatmulArgs a, int64_t B, hipStream_t st, void* workspace, siz
     // -- the general kernel reaches about 60 % of the pipelined one's rate -- and for a single
     // row of tiles from 129 rows on, where the general kernel would need two rows of its 128-row tiles)
     const int64_t m_pad = (a.M + 255) / 256 * 256;
+    // (97 ... 128 rows: the general kernel's single row of 128 x 128 tiles cannot split K; the padded
+    // pipelined kernel can, and wins when K is long -- 16:32: from K = 1024; dense: from K = 2048 on
+    // outputs too narrow to give the general kernel a tile per CU and a half)
+    const bool pad_97_128 = a.M > 96 && a.M <= 128 && (SPARSE ? a.K >= 1024 : (a.K >= 2048 && a.S <= 12288));
     // (the kernel addresses with 32-bit byte offsets into buffer resources: 256 rows of states,
     // the whole packed matrix and the whole of scales / zeros have to stay below 2 GB each)
     const int64_t w_bytes = (int64_t)a.K / 32 * PipeFmt<BITS, SPARSE>::ROWS * 4 * a.S;
     const int64_t sz_bytes = ((int64_t)a.K / 64 + a.group_units - 1) / a.group_units * a.S * 2;
-    const bool m_ok = (m_pad * 2 <= a.M * 3 || (a.M > 128 && a.M <= 256)) && a.K <= (1 << 22) && a.S <= (1 << 27) &&
+    const bool m_ok = (m_pad * 2 <= a.M * 3 || (a.M > 128 && a.M <= 256) || pad_97_128) && a.K <= (1 << 22) && a.S <= (1 << 27) &&
                       w_bytes < (1ll << 31) && sz_bytes < (1ll << 31);
     const bool pipe2_ok = !SPARSE && m_ok && a.S % 128 == 0;
     const bool pipe4_ok = m_ok && a.S % 256 == 0;
