@@ -577,7 +577,7 @@ __global__ __launch_bounds__(512) void skinny_kernel(SkinnyArgs a) {
     }
 }
 
-// ---- 33 ... 96 rows, dense formats: the eight waves of a workgroup share one staged copy of the states.
+// ---- 17 ... 256 rows, every format: the eight waves of a workgroup share one staged copy of the states.
 // In the kernel above every wave stages the states of its own units, so a workgroup of 64 columns reads
 // all R x K states: with R = 64 that is four times the packed weights it reads.  Here the waves stand side
 // by side along the columns (32 each, 256 per workgroup), all walk the same units, and each unit's states
@@ -588,9 +588,9 @@ __global__ __launch_bounds__(512) void skinny_kernel(SkinnyArgs a) {
 // dequantising each weight: the operand is the reference's fp16(fp16(q - z) s), three packed operations
 // per pair of weights on top of the magic-number decode, and the accumulators hold the product itself.
 // K is split across workgroups (blockIdx.z) with the hand-over above, one counter per wave.
-template <int BITS, int MT>
+template <int BITS, int MT, bool SPARSE = false>
 __global__ __launch_bounds__(512) void wide_rows_kernel(SkinnyArgs a) {
-    using F = SkFmt<BITS>;
+    using F = SkFmt<BITS, SPARSE>;
     constexpr int CW = 2, NL = F::LOADS, PF = 4, ROWS = 16 * MT, STRIP = 16 * CW, WSTRIP = 8 * STRIP;
     constexpr int XBUF = ROWS * SK_PITCH;
     extern __shared__ __attribute__((aligned(16))) char lds[];
@@ -606,6 +606,25 @@ __global__ __launch_bounds__(512) void wide_rows_kernel(SkinnyArgs a) {
     const int group_lo = u0 / a.group_units;
     const int groups = (u1 + a.group_units - 1) / a.group_units - group_lo;
 
+    // (16:32: the selector table of the kernel above, same layout)
+    __shared__ __attribute__((aligned(16))) u32x4 lut_table[SPARSE ? 256 : 1];
+    const char* lut = reinterpret_cast<const char*>(lut_table);
+    if constexpr (SPARSE) {
+        for (int b = t; b < 256; b += 512) {
+            uint32_t selb[8];
+            int rank = 0;
+#pragma unroll
+            for (int r = 0; r < 8; ++r) {
+                const bool k = (b >> r) & 1;
+                selb[r] = k ? (uint32_t)((rank & 1) * 4 + (rank >> 1)) : 0x0Cu;
+                rank += k;
+            }
+            u32x4 e;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) e[q] = selb[q] | (0x0Cu << 8) | (selb[q + 4] << 16) | (0x0Cu << 24);
+            lut_table[((b & 15) << 4) | (b >> 4)] = e;
+        }
+    }
     // LDS: two unit buffers, a flag, the strip's scales and zeros
     char* const xb = lds;
     int* const flag = reinterpret_cast<int*>(lds + 2 * XBUF);
@@ -637,13 +656,24 @@ __global__ __launch_bounds__(512) void wide_rows_kernel(SkinnyArgs a) {
     // weights of unit u: as in the kernel above (lane group h: chunk h of each of the unit's two blocks)
     const int wrow = BITS == 4 ? h : (h >> 1);
     const int wshift = BITS == 4 ? 0 : (BITS == 2 ? 16 * (h & 1) : (h == 0 ? 0 : h == 1 ? 24 : h == 2 ? 16 : 40));
-    const uint32_t* wbase = a.matrix + (int64_t)wrow * a.S + col0;
+    const uint32_t* wbase = a.matrix + (int64_t)(SPARSE ? 0 : wrow) * a.S + col0;
+    const uint32_t* mbase = SPARSE ? a.mask + col0 : nullptr;
     auto load_w = [&](words_t w[NL], int u) {
         const uint32_t* p = wbase + (int64_t)u * (2 * F::ROWS) * a.S;
+        if constexpr (SPARSE) {          // every lane group: both words of kept codes and the mask word of each block
+            const uint32_t* pm = mbase + (int64_t)u * 2 * a.S;
 #pragma unroll
-        for (int i = 0; i < NL; ++i) {
-            const int row = BITS == 3 ? 3 * (i >> 1) + (i & 1) : F::ROWS * i;
-            w[i] = __builtin_nontemporal_load(reinterpret_cast<const words_t*>(p + (int64_t)row * a.S));
+            for (int blk = 0; blk < 2; ++blk) {
+                w[3 * blk] = __builtin_nontemporal_load(reinterpret_cast<const words_t*>(p + (int64_t)(2 * blk) * a.S));
+                w[3 * blk + 1] = __builtin_nontemporal_load(reinterpret_cast<const words_t*>(p + (int64_t)(2 * blk + 1) * a.S));
+                w[3 * blk + 2] = __builtin_nontemporal_load(reinterpret_cast<const words_t*>(pm + (int64_t)blk * a.S));
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < NL; ++i) {
+                const int row = BITS == 3 ? 3 * (i >> 1) + (i & 1) : F::ROWS * i;
+                w[i] = __builtin_nontemporal_load(reinterpret_cast<const words_t*>(p + (int64_t)row * a.S));
+            }
         }
     };
     auto chunk_bits = [&](const words_t w[NL], int blk, int c) -> uint32_t {
@@ -687,6 +717,29 @@ __global__ __launch_bounds__(512) void wide_rows_kernel(SkinnyArgs a) {
             c2[c] = h16x2{ze[c], ze[c]};
         }
     };
+    // 16:32: the expanded chunk (halves 0x001q for a kept row, 0 for a dropped one; see the kernel above)
+    // ORed with 1024 is 1040 + q; minus 1040 the code, exactly, or -16; then the same two roundings, and
+    // the dropped rows are multiplied by 0 -- bit 4 of the half, the "kept" flag, times 0x3C0 is fp16 1.0
+    const uint32_t below = SPARSE ? (1u << (8 * h)) - 1u : 0u, rep_h = 0x01010101u * h;
+    const uint32_t sp_nib = SPARSE ? vgpr_const(0x0F0F0F0Fu) : 0u, sp_flag = SPARSE ? vgpr_const(0x10101010u) : 0u;
+    const uint32_t sp_kept = SPARSE ? vgpr_const(0x00100010u) : 0u, sp_idx = SPARSE ? vgpr_const(0x00000FF0u) : 0u;
+    auto sparse_chunk = [&](const words_t w[NL], int blk, int c, uint32_t& v, uint32_t& mb4) {
+        const uint32_t m = word_of<CW>(w[3 * blk + 2], c);
+        const uint64_t st = ((uint64_t)word_of<CW>(w[3 * blk + 1], c) << 32) | word_of<CW>(w[3 * blk], c);
+        v = (uint32_t)(st >> ((uint32_t)__builtin_popcount(m & below) << 2));
+        mb4 = __builtin_amdgcn_perm(m, m, rep_h);           // mask byte h, four times
+    };
+    auto sparse_scaled_operand = [&](uint32_t v, uint32_t mb4, int c) -> h16x8 {
+        const u32x4 sel = *reinterpret_cast<const u32x4*>(lut + (mb4 & sp_idx));
+        u32x4 r = sparse_operand(v, sel, sp_nib, sp_flag);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const h16x2 kept = as_h2((r[e] & sp_kept) * 0x3C0u);
+            const h16x2 q = as_h2(r[e] | 0x64006400u) - as_h2(0x64106410u);
+            r[e] = bitcast<uint32_t>(((q - c2[c]) * kept) * s2[c]);
+        }
+        return bitcast<h16x8>(r);
+    };
     // the chunk's magic numbers minus their offsets are the codes, exactly; then the reference's own
     // two roundings: fp16(fp16(q - z) s) (matmul.cuh:115-125)
     auto scaled_operand = [&](uint32_t f, int c) -> h16x8 {
@@ -722,8 +775,15 @@ __global__ __launch_bounds__(512) void wide_rows_kernel(SkinnyArgs a) {
                     xa[mt] = *reinterpret_cast<const h16x8*>(xb + p * XBUF + (j + 16 * mt) * SK_PITCH + (i * 4 + h) * 16);
 #pragma unroll
                 for (int c = 0; c < CW; ++c) {
-                    const uint32_t f = chunk_bits(wu, i, c);
-                    const h16x8 wb = general ? exact_operand<BITS>(f, sc[c], ze[c]) : scaled_operand(f, c);
+                    h16x8 wb;
+                    if constexpr (SPARSE) {
+                        uint32_t v, mb4;
+                        sparse_chunk(wu, i, c, v, mb4);
+                        wb = general ? exact_operand_sparse(v, mb4 & 0xFFu, sc[c], ze[c]) : sparse_scaled_operand(v, mb4, c);
+                    } else {
+                        const uint32_t f = chunk_bits(wu, i, c);
+                        wb = general ? exact_operand<BITS>(f, sc[c], ze[c]) : scaled_operand(f, c);
+                    }
 #pragma unroll
                     for (int mt = 0; mt < MT; ++mt)
                         acc[c][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[mt], wb, acc[c][mt], 0, 0, 0);
@@ -815,7 +875,7 @@ static WidePlan plan_wide(int64_t R, int64_t K, int64_t S, bool sparse) {
     WidePlan p{false, 0, 0, 0, 1, 0, 0};
     // (knob: 1 = never, n >= 2 = from n rows on whatever the shape)
     const int64_t knob = tuning(TUNE_NO_WIDE), min_rows = knob >= 2 ? knob : 17;
-    if (sparse || R < min_rows || R > SK_WIDE_MAX_ROWS || S % 256 != 0 || K % 64 != 0 || knob == 1) return p;
+    if (R < min_rows || R > SK_WIDE_MAX_ROWS || S % 256 != 0 || K % 64 != 0 || knob == 1) return p;
     p.row_blocks = (int)((R + 63) / 64);
     p.block_rows = (int)(((R + p.row_blocks - 1) / p.row_blocks + 15) / 16 * 16);
     p.mt = p.block_rows / 16;
@@ -833,23 +893,31 @@ static WidePlan plan_wide(int64_t R, int64_t K, int64_t S, bool sparse) {
     // measured against the kernel above (K = 2048 ... 20480, S = 1024 ... 28672): with 17 ... 32 rows it
     // needs wide matrices and long shares of K, with 33 ... 64 rows matrices of 32 M weights and more
     // and from 129 rows on the tile kernels win on wide outputs
+    // (16:32, whose decode costs more here and in the tile kernels alike: 17 ... 32 rows from 64 M weights
+    // on, 33 ... 64 rows from 32 M, 65 ... 128 rows always, beyond that for narrow outputs)
     if (knob < 2 && forced < 1) {
-        if (R <= 32 && (wgs < 32 || p.units_per_split < 16)) return p;
-        if (R > 32 && R <= 64 && K * S < (1ll << 25)) return p;
-        if (R > 128 && S > 8192) return p;
+        if (sparse) {
+            if (R <= 32 && K * S < (1ll << 26)) return p;
+            if (R > 32 && R <= 64 && K * S < (1ll << 25)) return p;
+            if (R > 128 && (S > 5120 || (R > 192 && S > 4096))) return p;
+        } else {
+            if (R <= 32 && (wgs < 32 || p.units_per_split < 16)) return p;
+            if (R > 32 && R <= 64 && K * S < (1ll << 25)) return p;
+            if (R > 128 && S > 8192) return p;
+        }
     }
     p.part_bytes = p.ksplit > 1 ? (size_t)wgs * 8 * p.ksplit * (2 * p.mt * 4 * 256) : 0;
     p.use = true;
     return p;
 }
 
-template <int BITS>
+template <int BITS, bool SPARSE = false>
 static bool launch_wide(SkinnyArgs a, const WidePlan& p, hipStream_t st) {
     const int upg = a.group_units;
     int groups = (a.K / 64 + upg - 1) / upg;
     if (p.ksplit > 1) groups = std::min(groups, (p.units_per_split + upg - 1) / upg + 1);
     const size_t lds = 2 * (size_t)p.block_rows * SK_PITCH + 1024 + 16 + (size_t)groups * 256 * 4;
-    if (lds > 150 * 1024) return false;
+    if (lds > 150 * 1024 - (SPARSE ? 4096 : 0)) return false;
     a.block_rows = p.block_rows;
     a.units_per_split = p.units_per_split;
     const dim3 grid((unsigned)(a.S / 256), (unsigned)p.row_blocks, (unsigned)p.ksplit), block(512);
@@ -864,10 +932,10 @@ static bool launch_wide(SkinnyArgs a, const WidePlan& p, hipStream_t st) {
         }
         hipLaunchKernelGGL(kernel, grid, block, lds, st, a);
     };
-    if (p.mt == 1) go(wide_rows_kernel<BITS, 1>, 0);
-    else if (p.mt == 2) go(wide_rows_kernel<BITS, 2>, 1);
-    else if (p.mt == 3) go(wide_rows_kernel<BITS, 3>, 2);
-    else go(wide_rows_kernel<BITS, 4>, 3);
+    if (p.mt == 1) go(wide_rows_kernel<BITS, 1, SPARSE>, 0);
+    else if (p.mt == 2) go(wide_rows_kernel<BITS, 2, SPARSE>, 1);
+    else if (p.mt == 3) go(wide_rows_kernel<BITS, 3, SPARSE>, 2);
+    else go(wide_rows_kernel<BITS, 4, SPARSE>, 3);
     return true;
 }
 
@@ -976,7 +1044,8 @@ bool skinny_rows(int bits, h16* outs, const uint32_t* matrix, const h16* x, cons
             a.units_per_wave = 0;
             a.counters = reinterpret_cast<int*>(ws.counters);
             a.part = reinterpret_cast<float*>(ws.scratch);
-            const bool ok = bits == 4 ? launch_wide<4>(a, wp, st) : bits == 3 ? launch_wide<3>(a, wp, st) : launch_wide<2>(a, wp, st);
+            const bool ok = sparse_mask ? launch_wide<4, true>(a, wp, st)
+                          : bits == 4 ? launch_wide<4>(a, wp, st) : bits == 3 ? launch_wide<3>(a, wp, st) : launch_wide<2>(a, wp, st);
             if (ok) return true;
         }
     }

@@ -271,3 +271,74 @@ def test_shared_staging_up_to_256_rows(H, bits, M, K, S, g):
     finally:
         H.capi.tune(8, 0)
     assert O.max_rel_error(ref.astype(np.float64), got) < H.TOL_EXACT_MTX
+
+
+# ---- 16:32 through the shared-staging kernel
+@pytest.mark.parametrize("M,K,S,g", [(17, 1024, 512, 64), (33, 2048, 256, 128), (64, 4096, 256, 64), (65, 1024, 1024, -1),
+                                     (96, 2048, 512, 64), (128, 4096, 256, 64), (200, 1024, 768, 128), (256, 2048, 512, 64),
+                                     (2, 512, 256, 64), (40, 64, 256, 64)])
+def test_shared_staging_sparse(H, M, K, S, g):
+    capi = H.capi
+    p = O.make_problem(bits=4, K=K, S=S, M=M, group_size=g, sparse=True, seed=M + K + S)
+    d = H.dev_problem(p)
+    exact, f32 = H.oracles(p)
+    runs = []
+    capi.tune(8, 2)                          # whatever the shape
+    try:
+        ws = capi.new_matmul_workspace(1, M, K, S, True)
+        for _ in range(2):
+            o = torch.full((1, M, S), 9.0, dtype=torch.float16, device="cuda")
+            capi.matmul(4, o, d["matrix"], d["states"], d["scales"], d["zeros"], g, d["mask"], ws)
+            torch.cuda.synchronize()
+            runs.append(o.cpu().numpy())
+    finally:
+        capi.tune(8, 0)
+    H.assert_product_close(runs[0], exact, f32, kind="mtx")       # (the reference's two roundings per weight)
+    assert np.array_equal(runs[0], runs[1])
+    capi.tune(8, 1)
+    try:
+        ref = H.run_capi(p, d, "mtx")
+    finally:
+        capi.tune(8, 0)
+    assert O.max_rel_error(ref.astype(np.float64), runs[0]) < H.TOL_EXACT
+
+
+def test_shared_staging_sparse_exponent_mode_batches_and_crowded_masks(H):
+    H.capi.tune(8, 2)
+    try:
+        p = O.make_problem(bits=4, K=2048, S=512, M=1, B=50, group_size=64, sparse=True, seed=31)
+        p["scales"][1, 40:48] *= np.float16(-1)
+        p["scales"][9, 300] *= np.float16(-1)
+        prior = np.random.default_rng(5).standard_normal((50, 1, 512)).astype(np.float16)
+        _check(H, p, "vec", prior=prior)              # the matvec entry adds onto outs
+        # masks whose kept rows crowd one end of a block
+        K, S, M = 256, 256, 40
+        rng = np.random.default_rng(3)
+        codes = rng.integers(0, 16, size=(K, S), dtype=np.uint8)
+        keep = np.zeros((K // 32, 32, S), dtype=bool)
+        keep[0, :16] = True
+        keep[1, 16:] = True
+        keep[2, 8:24] = True
+        keep[3, ::2] = True
+        keep[4, :8] = True
+        keep[4, 24:] = True
+        keep[5, 1::2] = True
+        keep[6, :4] = True
+        keep[6, 20:] = True
+        keep[7, 3:19] = True
+        keep = keep.reshape(K, S)
+        matrix, mask = O.sparse_pack(np.ascontiguousarray(codes.T), np.ascontiguousarray(keep.T).astype(np.uint8))
+        q = dict(B=1, M=M, S=S, K=K, bits=4, group_size=64, matrix=matrix, sparse_mask=mask, keep=keep,
+                 codes=np.where(keep, codes, np.uint8(0)), states=rng.standard_normal((1, M, K)).astype(np.float16),
+                 scales=rng.uniform(0.001, 0.02, size=(K // 64, S)).astype(np.float16),
+                 zeros=rng.uniform(0, 15, size=(K // 64, S)).astype(np.float16))
+        _check(H, q, "mtx")
+    finally:
+        H.capi.tune(8, 0)
+
+
+@pytest.mark.parametrize("M", [40, 100, 128])
+def test_shared_staging_sparse_default_rule(H, M):
+    """K=4096, S=8192 (32 M weights), 16:32: 33 rows and more take the shared-staging kernel by default"""
+    p = O.make_problem(bits=4, K=4096, S=8192, M=M, group_size=64, sparse=True, seed=M)
+    _check(H, p, "mtx")
