@@ -194,6 +194,23 @@ def main():
                                        "traffic": MATMUL_TRAFFIC_BYTES},
                           "max_rel_err_vs_fp32_oracle": float(f"{mm_err:.3e}")}
 
+        # ---- the few-row products in between (a batch of decoding requests): 8 and 64 rows, same weights
+        few = {}
+        for rows in (8, 64):
+            xr = xs[:, :rows].contiguous()
+            orow = torch.zeros((1, rows, S), dtype=torch.float16, device=dev)
+            ws_r = capi.new_matmul_workspace(1, rows, K, S)
+            us = timed(lambda: capi.matmul(4, orow, m, xr, sc, ze, g, None, ws_r), warm=10, batches=5, reps=20)
+            got_r = orow[0].cpu().numpy()
+            err_r = O.max_rel_error(O.matmul_fp32(xr[0].cpu().numpy(), w32), got_r)
+            assert err_r < 1e-2, f"{rows}-row product disagrees with the oracle: {err_r}"
+            nb = matvec_bytes(K, S, g) + 2 * rows * (K + S) - 2 * (K + S)
+            few[f"rows_{rows}"] = {"us": round(us, 2), "GB/s": round(nb / (us * 1e-6) / 1e9, 1),
+                                   "frac_of_hbm_peak": round(nb / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
+                                   "max_rel_err_vs_fp32_oracle": float(f"{err_r:.3e}")}
+        result["few_rows"] = {"workload": "int4 dense, K(N)=5120 S=20480 group=128, 8 and 64 rows of states "
+                                          "(weights warm in the last-level cache)", **few}
+
     # ---- CPU baseline: torch dequantise + fp32 matmul on the host (reported only)
     if not args.no_cpu:
         from oracle import cpu_baseline
