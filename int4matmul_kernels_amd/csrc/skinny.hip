@@ -1,6 +1,8 @@
-// Few-row product for gfx950: 2 .. 96 rows of states (32 per workgroup) against a dense int4 / int3 / int2
-// or 16:32 sparse int4 weight matrix, HBM-bound like the matvec (every packed word is read once and
-// used for all rows).  The reference has no such path: it sends M >= 2 to its
+// Few-row products for gfx950, two kernels.  skinny_kernel (described first): 2 .. 96 rows of states (32 per
+// workgroup) against a dense int4 / int3 / int2 or 16:32 sparse int4 weight matrix, HBM-bound like the
+// matvec (every packed word is read once and used for all rows).  wide_rows_kernel (further down): 17 .. 256
+// rows, whose waves share one staged copy of the states and dequantise each weight.  skinny_rows() at the
+// end picks one by shape.  The reference has no such path: it sends M >= 2 to its
 // 64-row matmul tiles (int4matmul.cpp:27) and M == 1 with B > 1 to one matvec
 // per batch element, re-reading the weights each time (matvec_kernel.cu:346).
 //
@@ -24,7 +26,7 @@
 // of CW adjacent columns: CW * 64 contiguous bytes per packed row and wave) and
 // its W waves split K; each wave stages the states of its own K range through
 // a private LDS buffer, 64 k at a time, and the partial tiles are summed
-// through LDS at the end -- no exchange between workgroups.
+// through LDS at the end; narrow matrices with a long K are also split along K across workgroups.
 //
 // 16:32 sparse int4 takes the same kernel.  Every lane group loads the block's
 // mask word and both words of kept codes (the four groups of a wave ask for the
