@@ -915,10 +915,10 @@ constexpr int64_t MM_SPLIT_MAX_BYTES = 192ll << 20;      // cap of the partial t
 struct SplitPlan { int ksplit; int64_t tiles; int64_t tile_bytes; };
 static SplitPlan plan_split(bool sparse, int64_t B, int64_t M, int64_t K, int64_t S) {
     const SplitPlan none{1, 0, 0};
-    if (S % 256 != 0) return none;
-    const int64_t m_pad = (M + 255) / 256 * 256, tiles4 = m_pad / 256 * (S / 256) * B;
+    if (S % (sparse ? 256 : 128) != 0) return none;
+    const int64_t m_pad = (M + 255) / 256 * 256, tiles4 = m_pad / 256 * ((S + 255) / 256) * B;
     if (tiles4 > 128) return none;
-    SplitPlan p{1, sparse ? tiles4 : 2 * tiles4, sparse ? 256 * 256 * 4 : 256 * 128 * 4};
+    SplitPlan p{1, m_pad / 256 * (S / (sparse ? 256 : 128)) * B, sparse ? 256 * 256 * 4 : 256 * 128 * 4};
     if (p.tiles > MM_SPLIT_MAX_TILES) return none;
     const int64_t steps = K / 32, forced = tuning(TUNE_MM_SPLIT);
     auto cost = [&](int64_t ks) { return (p.tiles * ks + 255) / 256 * ((steps + ks - 1) / ks + 20) + (ks > 1 ? 6 * ks : 0); };
@@ -991,10 +991,13 @@ static void launch(MatmulArgs a, int64_t B, hipStream_t st, void* workspace, siz
     const bool tail_ok = pipe4_ok && tp.ksplit > 1 && wsp.counters != nullptr &&
                          wsp.scratch_bytes >= (size_t)(tp.tiles * tp.ksplit * (256 * 256 * 4));
     if (variant == 0) {
-        const int64_t tiles4 = m_pad / 256 * (a.S / 256) * B;
+        const int64_t tiles4 = m_pad / 256 * ((a.S + 255) / 256) * B;
         const int64_t last = tiles4 % 256;
         const bool small_better = tiles4 <= 128 || (!tail_ok && tiles4 > 256 && tiles4 < 512 && last > 0 && last <= 96);
-        if (pipe4_ok && (SPARSE || !pipe2_ok || !small_better)) variant = 6;
+        // (a grid that fills at most half of the GPU with a short K: the pipelined kernel's prologue -- three
+        // stages, the scan of the scales -- costs more than its faster steps return; measured K <= 1024)
+        if (!SPARSE && tiles4 <= 128 && a.K <= 1024) variant = 1;
+        else if (pipe4_ok && (SPARSE || !pipe2_ok || !small_better)) variant = 6;
         else if (pipe2_ok) variant = 5;
         else if (a.M > 512 && a.S >= 256) variant = 3;
         else variant = 1;
