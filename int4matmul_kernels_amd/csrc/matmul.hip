@@ -978,12 +978,23 @@ static void launch(MatmulArgs a, int64_t B, hipStream_t st, void* workspace, siz
     // the whole packed matrix and the whole of scales / zeros have to stay below 2 GB each)
     const int64_t w_bytes = (int64_t)a.K / 32 * PipeFmt<BITS, SPARSE>::ROWS * 4 * a.S;
     const int64_t sz_bytes = ((int64_t)a.K / 64 + a.group_units - 1) / a.group_units * a.S * 2;
-    const bool m_ok = (m_pad * 2 <= a.M * 3 || (a.M > 128 && a.M <= 256) || pad_97_128) && a.K <= (1 << 22) && a.S <= (1 << 27) &&
-                      w_bytes < (1ll << 31) && sz_bytes < (1ll << 31);
+    const bool shape_ok = a.K <= (1 << 22) && a.S <= (1 << 27) && w_bytes < (1ll << 31) && sz_bytes < (1ll << 31);
+    // (257 ... 341 rows, padded by half and more: still better than the general kernel where split-K makes up
+    // for a small grid, and for 16:32 everywhere -- its general decode is slow; measured K >= 2048)
+    const bool pad_257_341 = a.M > 256 && a.M < 342 && a.K >= 2048 &&
+                             (SPARSE || m_pad / 256 * ((a.S + 255) / 256) * B <= 128);
+    const bool m_ok = (m_pad * 2 <= a.M * 3 || (a.M > 128 && a.M <= 256) || pad_97_128 || pad_257_341) && shape_ok;
+    // 257 ... 384 rows: three rows of 128 x 256 tiles (the same kernel with half the rows per wave) instead of
+    // two rows of 256 x 256 padded by a quarter and more -- when they give the GPU at most one round of at
+    // least half (16:32: three quarters) of its CUs; smaller grids are better off with split-K
+    const int64_t tiles_128 = (a.M + 127) / 128 * (a.S / 256) * B;
+    const bool three_rows = a.M > 256 && a.M <= 384 && shape_ok && a.S % 256 == 0 && tiles_128 <= 256 &&
+                            tiles_128 >= (SPARSE ? 192 : 128);
     const bool pipe2_ok = !SPARSE && m_ok && a.S % 128 == 0;
     const bool pipe4_ok = m_ok && a.S % 256 == 0;
-    if (variant != 1 && variant != 3 && variant != 5 && variant != 6 && variant != 9) variant = 0;
-    if ((variant == 5 && !pipe2_ok) || ((variant == 6 || variant == 9) && !pipe4_ok)) variant = 0;
+    if (variant != 1 && variant != 3 && variant != 5 && variant != 6 && variant != 7 && variant != 9) variant = 0;
+    if ((variant == 5 && !pipe2_ok) || ((variant == 6 || variant == 9) && !pipe4_ok) ||
+        (variant == 7 && !(shape_ok && a.S % 256 == 0))) variant = 0;
     // (a last round of large tiles that fills at most half of the GPU is split along K when the
     // workspace has room for its partial tiles: better than small tiles then)
     const TailPlan tp = plan_tail(B, a.M, a.K, a.S);
@@ -997,6 +1008,7 @@ static void launch(MatmulArgs a, int64_t B, hipStream_t st, void* workspace, siz
         // (a grid that fills at most half of the GPU with a short K: the pipelined kernel's prologue -- three
         // stages, the scan of the scales -- costs more than its faster steps return; measured K <= 1024)
         if (!SPARSE && tiles4 <= 128 && a.K <= 1024) variant = 1;
+        else if (three_rows) variant = 7;
         else if (pipe4_ok && (SPARSE || !pipe2_ok || !small_better)) variant = 6;
         else if (pipe2_ok) variant = 5;
         else if (a.M > 512 && a.S >= 256) variant = 3;
@@ -1024,6 +1036,7 @@ static void launch(MatmulArgs a, int64_t B, hipStream_t st, void* workspace, siz
     else if (variant == 3) launch_tile<BITS, SPARSE, 128, 256, 128, 64>(a, B, st);
     // (256 x 256: the dense formats run the two halves of the workgroup in opposite phases, 2-3 %
     // faster; the 16:32 decode has no registers to spare for it.  Variant 9 forces the plain order.)
+    else if (variant == 7) launch_pipe<BITS, SPARSE, 4, 2>(a, B, st);
     else if (variant == 6 && !SPARSE) launch_pipe<BITS, SPARSE, 4, 4, true>(a, B, st);
     else if (variant == 6 || variant == 9) launch_pipe<BITS, SPARSE, 4>(a, B, st);
     else if constexpr (!SPARSE) launch_pipe<BITS, false, 2>(a, B, st);

@@ -215,3 +215,43 @@ def test_pipelined_matmul_with_exponent_groups(H, bits, sparse, variant, M, K, S
         H.assert_product_close(H.run_capi(p, d, "mtx"), exact, f32, kind="mtx")
     finally:
         capi.tune(3, 0)
+
+
+# ---- 257 ... 384 rows: three rows of 128 x 256 tiles of the pipelined kernel (tuning key 3 = 7 forces them), and the
+# padded 256-row tiles that serve 257 ... 341 rows on small grids and for 16:32
+@pytest.mark.parametrize("bits,sparse", FORMATS)
+@pytest.mark.parametrize("M,K,S,g", [(384, 512, 512, 128), (300, 2048, 256, 64), (257, 1024, 768, -1), (341, 2560, 256, 128)])
+def test_matmul_three_rows_of_128_row_tiles(H, bits, sparse, M, K, S, g):
+    p = _problem(bits, sparse, K=K, S=S, M=M, group_size=g, seed=M + S)
+    d = H.dev_problem(p)
+    exact, f32 = H.oracles(p)
+    H.capi.tune(8, 1)            # (not the few-row path)
+    try:
+        auto = H.run_capi(p, d, "mtx", outs_init=np.full((1, M, S), 4.0, np.float16))
+        H.assert_product_close(auto, exact, f32, kind="mtx")
+        H.capi.tune(3, 7)
+        try:
+            got = H.run_capi(p, d, "mtx", outs_init=np.full((1, M, S), 4.0, np.float16))
+        finally:
+            H.capi.tune(3, 0)
+    finally:
+        H.capi.tune(8, 0)
+    H.assert_product_close(got, exact, f32, kind="mtx")
+    assert O.max_rel_error(auto.astype(np.float64), got) < H.TOL_EXACT_MTX
+
+
+@pytest.mark.parametrize("bits,sparse", [(4, False), (4, True)])
+def test_matmul_three_rows_default_rule_and_exponent_groups(H, bits, sparse):
+    """M=300 against S=11264 (44 tile columns: 132 tiles of 128 x 256) takes the variant by default for the dense
+    format; some exponent-mode groups on top"""
+    p = _problem(bits, sparse, K=1024, S=11264, M=300, group_size=128, seed=12)
+    p["scales"][2, 100:108] *= np.float16(-1)
+    p["scales"][5, 7000] *= np.float16(-1)
+    d = H.dev_problem(p)
+    exact, f32 = H.oracles(p)
+    H.capi.tune(8, 1)
+    try:
+        got = H.run_capi(p, d, "mtx")
+    finally:
+        H.capi.tune(8, 0)
+    H.assert_product_close(got, exact, f32, kind="mtx")
