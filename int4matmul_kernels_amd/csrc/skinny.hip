@@ -901,6 +901,7 @@ static WidePlan plan_wide(int64_t R, int64_t K, int64_t S, bool sparse) {
         if (sparse) {
             if (R <= 32 && K * S < (1ll << 26)) return p;
             if (R > 32 && R <= 64 && K * S < (1ll << 25)) return p;
+            if (R > 96 && R <= 128 && S > 16384) return p;       // (the padded 256-row tiles win on very wide outputs)
             if (R > 128 && (S > 5120 || (R > 192 && S > 4096))) return p;
         } else {
             if (R <= 32 && (wgs < 32 || p.units_per_split < 16)) return p;
