@@ -893,7 +893,7 @@ static WidePlan plan_wide(int64_t R, int64_t K, int64_t S, bool sparse) {
     p.units_per_split = (int)((units + ks - 1) / ks);
     p.ksplit = (int)((units + p.units_per_split - 1) / p.units_per_split);
     // measured against the kernel above (K = 2048 ... 20480, S = 1024 ... 28672): with 17 ... 32 rows it
-    // needs wide matrices and long shares of K, with 33 ... 64 rows matrices of 32 M weights and more
+    // needs 32 ... 96 strips and long shares of K, with 33 ... 64 rows matrices of 32 M weights and more
     // and from 129 rows on the tile kernels win on wide outputs
     // (16:32, whose decode costs more here and in the tile kernels alike: 17 ... 32 rows from 64 M weights
     // on, 33 ... 64 rows from 32 M, 65 ... 128 rows always, beyond that for narrow outputs)
@@ -904,7 +904,7 @@ static WidePlan plan_wide(int64_t R, int64_t K, int64_t S, bool sparse) {
             if (R > 96 && R <= 128 && S > 16384) return p;       // (the padded 256-row tiles win on very wide outputs)
             if (R > 128 && (S > 5120 || (R > 192 && S > 4096))) return p;
         } else {
-            if (R <= 32 && (wgs < 32 || p.units_per_split < 16)) return p;
+            if (R <= 32 && (wgs < 32 || wgs > 96 || p.units_per_split < 16)) return p;
             if (R > 32 && R <= 64 && K * S < (1ll << 25)) return p;
             if (R > 128 && S > 8192) return p;
         }
