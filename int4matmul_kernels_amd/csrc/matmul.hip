@@ -984,12 +984,13 @@ static void launch(MatmulArgs a, int64_t B, hipStream_t st, void* workspace, siz
     const bool pad_257_341 = a.M > 256 && a.M < 342 && a.K >= 2048 &&
                              (SPARSE || m_pad / 256 * ((a.S + 255) / 256) * B <= 128);
     const bool m_ok = (m_pad * 2 <= a.M * 3 || (a.M > 128 && a.M <= 256) || pad_97_128 || pad_257_341) && shape_ok;
-    // 257 ... 384 rows: three rows of 128 x 256 tiles (the same kernel with half the rows per wave) instead of
-    // two rows of 256 x 256 padded by a quarter and more -- when they give the GPU at most one round of at
-    // least half (16:32: three quarters) of its CUs; smaller grids are better off with split-K
-    const int64_t tiles_128 = (a.M + 127) / 128 * (a.S / 256) * B;
-    const bool three_rows = a.M > 256 && a.M <= 384 && shape_ok && a.S % 256 == 0 && tiles_128 <= 256 &&
-                            tiles_128 >= (SPARSE ? 192 : 128);
+    // An odd number of 128-row tile rows (257 ... 384 rows, 513 ... 640, ... up to 1152): 128 x 256 tiles (the
+    // same kernel with half the rows per wave) instead of 256 x 256 tiles padded by another 128 rows -- when
+    // they give the GPU at most one round of at least half (16:32: three quarters) of its CUs; smaller grids
+    // are better off with split-K
+    const int64_t rows_128 = (a.M + 127) / 128, tiles_128 = rows_128 * (a.S / 256) * B;
+    const bool three_rows = a.M > 256 && rows_128 % 2 == 1 && rows_128 <= 9 && shape_ok && a.S % 256 == 0 &&
+                            tiles_128 <= 256 && tiles_128 >= (SPARSE ? 192 : 128);
     const bool pipe2_ok = !SPARSE && m_ok && a.S % 128 == 0;
     const bool pipe4_ok = m_ok && a.S % 256 == 0;
     if (variant != 1 && variant != 3 && variant != 5 && variant != 6 && variant != 7 && variant != 9) variant = 0;

@@ -255,3 +255,13 @@ def test_matmul_three_rows_default_rule_and_exponent_groups(H, bits, sparse):
     finally:
         H.capi.tune(8, 0)
     H.assert_product_close(got, exact, f32, kind="mtx")
+
+
+@pytest.mark.parametrize("bits,sparse", [(4, False), (3, False), (4, True)])
+def test_matmul_five_rows_of_128_row_tiles_default_rule(H, bits, sparse):
+    """M=600 (five tile rows of 128) against S=11264: 220 tiles of 128 x 256, taken by default"""
+    p = _problem(bits, sparse, K=512, S=11264, M=600, group_size=64, seed=15)
+    d = H.dev_problem(p)
+    exact, f32 = H.oracles(p)
+    got = H.run_capi(p, d, "mtx", outs_init=np.full((1, 600, 11264), 4.0, np.float16))
+    H.assert_product_close(got, exact, f32, kind="mtx")
