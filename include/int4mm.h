@@ -75,7 +75,9 @@ INT4MM_API int int4mm_abi_version(void);
  * matmul and few-row kernels (1 = never split, 2..8 = that factor where the
  * shape allows a split at all), 7 = 1: the tiles of a matmul's last, partly
  * filled round are not split, 8 = the few-row kernel whose waves share the
- * staged states: 1 = never, n >= 2 = from n rows on whatever the shape. */
+ * staged states: 1 = never, n >= 2 = from n rows on whatever the shape,
+ * 9 = address of a device buffer of int64 [workgroups][8][16]: the dense int4 matvec then runs
+ * its instrumented variant and records time stamps there (see matvec_timeline.py). */
 INT4MM_API int int4mm_tune(int key, int64_t value);
 
 /* Shape of one product.  matrix_rows = R, n_groups = G (rows of scales/zeros).

@@ -89,7 +89,7 @@ int validate_product(int bits, const void* outs, const void* matrix, const void*
                      const int4mm_shape* sh, bool matvec);
 int64_t tuning(int key);                       // see int4mm_tune
 enum TuneKey { TUNE_MV_WAVES = 0, TUNE_MV_UNITS = 1, TUNE_MV_LK = 2, TUNE_MM_VARIANT = 3, TUNE_MV_NOPF = 4,
-               TUNE_NO_SKINNY = 5, TUNE_MM_SPLIT = 6, TUNE_MM_TAIL = 7, TUNE_NO_WIDE = 8, TUNE_COUNT = 9 };
+               TUNE_NO_SKINNY = 5, TUNE_MM_SPLIT = 6, TUNE_MM_TAIL = 7, TUNE_NO_WIDE = 8, TUNE_MV_TIMELINE = 9, TUNE_COUNT = 10 };
 
 // few-row product (2 .. 96 rows; sparse_mask != nullptr: 16:32 int4); false = shape not taken, use the general kernels
 bool skinny_rows(int bits, _Float16* outs, const uint32_t* matrix, const _Float16* x, const _Float16* scales,

@@ -50,6 +50,7 @@ struct MatvecArgs {
     int units_per_wg;
     int group_units;        // group size in units (>= 1); huge for a single group
     int splits;             // == gridDim.y
+    uint64_t* timeline;     // instrumented variant only: 16 time stamps per wave (8 wave slots per workgroup)
 };
 
 // ------------------------------------------------------------------ formats
@@ -371,7 +372,12 @@ __device__ __forceinline__ uint64_t slot_load(const uint64_t* p) {
 // PF: keep the next unit's loads in flight while the current one is processed
 // (more registers); without it a lane group loads and processes one unit at a
 // time and relies on the other resident waves to cover the latency.
-template <int BITS, bool SPARSE, int LK, bool PF>
+//
+// TL: instrumented variant (dense int4 only) that records, per wave, the 100 MHz wall clock at
+// entry (0), after its first requests (1), after the staging barrier (2), after each of its first
+// nine units (3..11), after the workgroup's reduction (12) and at the end (13), and the hardware
+// ids of where it ran (15).
+template <int BITS, bool SPARSE, int LK, bool PF, bool TL = false>
 __global__ __launch_bounds__(MV_MAX_WAVES * WAVE)
 void matvec_kernel(MatvecArgs a) {
     constexpr bool FAST = Fmt<BITS, SPARSE>::FAST;
@@ -391,6 +397,17 @@ void matvec_kernel(MatvecArgs a) {
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6, nwaves = blockDim.x >> 6;
     const int cl = lane % LC, kl = lane / LC;
     const int strip = blockIdx.x, split = blockIdx.y;
+    int stamped_units = 0;
+    auto stamp = [&](int k) {
+        if constexpr (TL) {
+            __builtin_amdgcn_sched_barrier(0);
+            uint64_t c = wall_clock64();
+            if (k == 15) c = ((uint64_t)__builtin_amdgcn_s_getreg((31 << 11) | 20) << 32) | __builtin_amdgcn_s_getreg((31 << 11) | 4);
+            if (lane == 0) a.timeline[((int64_t)(blockIdx.y * gridDim.x + blockIdx.x) * MV_MAX_WAVES + wave) * 16 + k] = c;
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    stamp(0);
     const int col = strip * COLS + cl * 4;
     const bool col_ok = col < a.S;
 
@@ -428,6 +445,7 @@ void matvec_kernel(MatvecArgs a) {
     if constexpr (PF) {
         if (work_b) load_unit(ub, a, u + ng, col);
     }
+    stamp(1);
 
     if constexpr (SPARSE) {
         // selector table: for mask byte b, pair j = (row j, row j+4): byte 0 picks the code of
@@ -532,6 +550,7 @@ void matvec_kernel(MatvecArgs a) {
         }
         __syncthreads();
     }
+    stamp(2);
 
     float y[4] = {0.f, 0.f, 0.f, 0.f};
     bool need_general = false;
@@ -585,11 +604,13 @@ void matvec_kernel(MatvecArgs a) {
             bool has_b = work_b;
             for (;;) {
                 finish_unit(ua, u);
+                if (stamped_units < 9) stamp(3 + stamped_units++);
                 if (!has_b) break;
                 const int u2 = u + 2 * ng, u3 = u + 3 * ng;
                 const bool has_a = u2 < wg_u1;
                 if (has_a) load_unit(ua, a, u2, col);
                 finish_unit(ub, u + ng);
+                if (stamped_units < 9) stamp(3 + stamped_units++);
                 if (!has_a) break;
                 has_b = u3 < wg_u1;
                 if (has_b) load_unit(ub, a, u3, col);
@@ -598,6 +619,7 @@ void matvec_kernel(MatvecArgs a) {
         } else {
             for (;;) {
                 finish_unit(ua, u);
+                if (stamped_units < 9) stamp(3 + stamped_units++);
                 u += ng;
                 if (u >= wg_u1) break;
                 load_unit(ua, a, u, col);
@@ -639,6 +661,7 @@ void matvec_kernel(MatvecArgs a) {
                 for (int k = 0; k < LK; ++k) total[i] += red[(w * 64 + k * LC) * 4 + j];
         }
     }
+    stamp(12);
     auto for_owned = [&](auto&& fn) {
 #pragma unroll
         for (int i = 0; i < MAXC; ++i) {
@@ -649,6 +672,7 @@ void matvec_kernel(MatvecArgs a) {
     };
     if (a.splits == 1) {
         for_owned([&](int i, int ocol) { a.outs[ocol] = (h16)((float)a.outs[ocol] + total[i]); });
+        stamp(13); stamp(15);
         return;
     }
 
@@ -659,6 +683,7 @@ void matvec_kernel(MatvecArgs a) {
     // next call and writes the result.
     if (split != a.splits - 1) {
         for_owned([&](int i, int ocol) { slot_store(&a.slots[(int64_t)split * a.S + ocol], total[i], SLOT_FULL); });
+        stamp(13); stamp(15);
         return;
     }
     for_owned([&](int i, int ocol) {
@@ -691,13 +716,19 @@ void matvec_kernel(MatvecArgs a) {
         // poisons the output instead of hanging the wave
         a.outs[ocol] = ok ? (h16)sum : (h16)__builtin_nanf("");
     });
+    stamp(13); stamp(15);
 }
 
 template <int BITS, bool SPARSE>
 static void launch(const MatvecArgs& a, int lk, bool pf, dim3 grid, dim3 block, hipStream_t st) {
     size_t lds = (size_t)a.units_per_wg * (Fmt<BITS, SPARSE>::XS + 8);     // staged states + per-unit sums
     if (lds < (size_t)block.x * 16) lds = (size_t)block.x * 16;           // reduction area: 4 floats per thread
-#define I4_LAUNCH(LK_, PF_) hipLaunchKernelGGL((matvec_kernel<BITS, SPARSE, LK_, PF_>), grid, block, lds, st, a)
+#define I4_LAUNCH(LK_, PF_) do { \
+        if constexpr (BITS == 4 && !SPARSE) { \
+            if (a.timeline) { hipLaunchKernelGGL((matvec_kernel<BITS, SPARSE, LK_, PF_, true>), grid, block, lds, st, a); break; } \
+        } \
+        hipLaunchKernelGGL((matvec_kernel<BITS, SPARSE, LK_, PF_, false>), grid, block, lds, st, a); \
+    } while (0)
     if (lk == 1) { if (pf) I4_LAUNCH(1, true); else I4_LAUNCH(1, false); }
     else if (lk == 2) { if (pf) I4_LAUNCH(2, true); else I4_LAUNCH(2, false); }
     else { if (pf) I4_LAUNCH(4, true); else I4_LAUNCH(4, false); }
@@ -708,10 +739,10 @@ static void launch(const MatvecArgs& a, int lk, bool pf, dim3 grid, dim3 block, 
 
 using namespace i4;
 
-extern "C" int int4mm_matvec(int bits, void* outs, const void* matrix, const void* multiplier,
-                             const void* scales, const void* zeros, const void* sparse_mask,
-                             const int4mm_shape* shape, void* workspace, size_t workspace_bytes,
-                             void* stream) {
+static int matvec_impl(int bits, void* outs, const void* matrix, const void* multiplier,
+                       const void* scales, const void* zeros, const void* sparse_mask,
+                       const int4mm_shape* shape, void* workspace, size_t workspace_bytes,
+                       void* stream) {
     int rc = validate_product(bits, outs, matrix, multiplier, scales, zeros, sparse_mask, shape, true);
     if (rc != INT4MM_OK) return rc;
     const int64_t B = shape->batch, K = shape->in_size, S = shape->out_size;
@@ -772,6 +803,7 @@ extern "C" int int4mm_matvec(int bits, void* outs, const void* matrix, const voi
     a.units_per_wg = upwg;
     a.group_units = (int)(g / 64 > 0x7FFFFFF ? 0x7FFFFFF : g / 64);
     a.splits = splits;
+    a.timeline = (uint64_t*)(uintptr_t)tuning(TUNE_MV_TIMELINE);
 
     const dim3 grid(strips, splits, 1), block(waves * WAVE);
     hipStream_t st = (hipStream_t)stream;
@@ -786,4 +818,11 @@ extern "C" int int4mm_matvec(int bits, void* outs, const void* matrix, const voi
         if (rc != INT4MM_OK) return rc;
     }
     return INT4MM_OK;
+}
+
+extern "C" int int4mm_matvec(int bits, void* outs, const void* matrix, const void* multiplier,
+                             const void* scales, const void* zeros, const void* sparse_mask,
+                             const int4mm_shape* shape, void* workspace, size_t workspace_bytes,
+                             void* stream) {
+    return matvec_impl(bits, outs, matrix, multiplier, scales, zeros, sparse_mask, shape, workspace, workspace_bytes, stream);
 }
