@@ -129,6 +129,21 @@ INT4MM_API int int4mm_matvec(int bits, void* outs, const void* matrix, const voi
                   const int4mm_shape* shape, void* workspace, size_t workspace_bytes,
                   void* stream);
 
+/* int4mm_matvec for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc): same arguments without
+ * the workspace, same kernels, same results bit for bit.  The hand-over slots and split-K
+ * partials live in a 16.8 MB device array built into the library (each GPU the library
+ * runs on holds its copy until the process ends), which covers out_size <= 32768; a wider
+ * product returns INT4MM_ERR_WORKSPACE.  The call allocates and frees nothing.  Its first
+ * call on a device looks up that device's copy of the array (make it once outside any
+ * graph capture).  All calls on one GPU share the array: calls that overlap in time on one
+ * GPU (two streams) race, exactly as two int4mm_matvec calls sharing one workspace would.
+ * No counterpart in the reference, whose matvec allocates an fp32 temporary per call
+ * (matvec_kernel.cu:351). */
+INT4MM_API int int4mm_matvec_static(int bits, void* outs, const void* matrix, const void* multiplier,
+                  const void* scales, const void* zeros, const void* sparse_mask,
+                  const int4mm_shape* shape, void* stream);
+
 /* Matrix-matrix product:
  *     outs[b,m,:] = fp16( sum_k fp32(multiplier[b,m,k]) * fp32(W[k,:]) )   (overwrites outs)
  * Replaces matmul_packed_int<bits> / matmul_int{4,3,2}

@@ -15,6 +15,7 @@ LIB_NAME = "libint4mm_hip.so"
 EXPORTS = [
     "int4mm_error_string", "int4mm_last_hip_error", "int4mm_abi_version", "int4mm_tune",
     "int4mm_workspace_bytes", "int4mm_workspace_init", "int4mm_matmul_workspace_bytes", "int4mm_matvec", "int4mm_matmul",
+    "int4mm_matvec_static",
     "int4mm_sparse_pack", "int4mm_dense_pack", "int4mm_unpack", "int4mm_dequantize",
 ]
 
@@ -61,6 +62,8 @@ def lib():
         f = getattr(L, name)
         f.restype = C.c_int
         f.argtypes = [C.c_int, vp, vp, vp, vp, vp, vp, C.POINTER(Shape), vp, sz, vp]
+    L.int4mm_matvec_static.restype = C.c_int
+    L.int4mm_matvec_static.argtypes = [C.c_int, vp, vp, vp, vp, vp, vp, C.POINTER(Shape), vp]
     L.int4mm_sparse_pack.restype = C.c_int
     L.int4mm_sparse_pack.argtypes = [vp, vp, vp, vp, i64, i64, vp, vp]
     L.int4mm_dense_pack.restype = C.c_int
@@ -120,6 +123,13 @@ def matvec(bits, outs, matrix, multiplier, scales, zeros, group_size, sparse_mas
     _check(lib().int4mm_matvec(bits, _ptr(outs), _ptr(matrix), _ptr(multiplier), _ptr(scales),
                                _ptr(zeros), _ptr(sparse_mask), C.byref(sh), _ptr(workspace), nws,
                                _stream()), "int4mm_matvec")
+
+
+def matvec_static(bits, outs, matrix, multiplier, scales, zeros, group_size, sparse_mask=None):
+    """the matvec that allocates nothing: scratch is a device array built into the library"""
+    sh = _shape(outs, matrix, multiplier, scales, group_size)
+    _check(lib().int4mm_matvec_static(bits, _ptr(outs), _ptr(matrix), _ptr(multiplier), _ptr(scales),
+                                      _ptr(zeros), _ptr(sparse_mask), C.byref(sh), _stream()), "int4mm_matvec_static")
 
 
 def matmul(bits, outs, matrix, multiplier, scales, zeros, group_size, sparse_mask=None, workspace=None):

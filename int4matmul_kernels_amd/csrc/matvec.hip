@@ -31,6 +31,8 @@
 // slots.  No cache-wide fence and no read-modify-write atomics are used.
 #include "common.h"
 
+#include <mutex>
+
 namespace i4 {
 
 constexpr int MV_MAX_WAVES = 8;
@@ -825,4 +827,41 @@ extern "C" int int4mm_matvec(int bits, void* outs, const void* matrix, const voi
                              const int4mm_shape* shape, void* workspace, size_t workspace_bytes,
                              void* stream) {
     return matvec_impl(bits, outs, matrix, multiplier, scales, zeros, sparse_mask, shape, workspace, workspace_bytes, stream);
+}
+
+// ---- the same product for callers that cannot allocate.  The hand-over slots and split-K
+// partials live in a file-scope device array instead of a caller's workspace.  Every device has
+// its own copy of the array at its own address, resolved once per device (with that device
+// current) and used from then on; host code never passes the array's name to a kernel.
+namespace i4 {
+constexpr int64_t STATIC_MAX_OUT_SIZE = 32768;
+// == int4mm_workspace_bytes(STATIC_MAX_OUT_SIZE): slots for 32 K splits x 32768 columns, the counter
+// page, and as much again as scratch for partial tiles
+constexpr size_t STATIC_SCRATCH_BYTES = 2 * (4096 + (size_t)STATIC_MAX_OUT_SIZE * 8 * 32 + 4096);
+static __device__ __align__(256) unsigned char scratch[STATIC_SCRATCH_BYTES];   // zero at load; calls leave it zeroed where it must be
+constexpr int STATIC_MAX_DEVICES = 64;
+static void* g_scratch_ptr[STATIC_MAX_DEVICES];
+static std::mutex g_scratch_mu;
+}  // namespace i4
+
+extern "C" int int4mm_matvec_static(int bits, void* outs, const void* matrix, const void* multiplier,
+                                    const void* scales, const void* zeros, const void* sparse_mask,
+                                    const int4mm_shape* shape, void* stream) {
+    if (shape == nullptr) return INT4MM_ERR_NULL;
+    if (shape->out_size > STATIC_MAX_OUT_SIZE) return INT4MM_ERR_WORKSPACE;     // beyond the built-in scratch
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= STATIC_MAX_DEVICES) return INT4MM_ERR_LAUNCH;
+    void* ptr;
+    {
+        std::lock_guard<std::mutex> lock(g_scratch_mu);
+        ptr = g_scratch_ptr[dev];
+        if (ptr == nullptr) {                                   // first call on this device
+            if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || ptr == nullptr) {
+                (void)hipGetLastError();
+                return INT4MM_ERR_LAUNCH;
+            }
+            g_scratch_ptr[dev] = ptr;
+        }
+    }
+    return matvec_impl(bits, outs, matrix, multiplier, scales, zeros, sparse_mask, shape, ptr, STATIC_SCRATCH_BYTES, stream);
 }
