@@ -10,9 +10,10 @@ Every function cites the reference lines it follows (paths relative to the
 reference checkout).  How each function is pinned independently of its own
 formula is listed beside it ("pinned by").  ``dequant_exponent`` and the
 negative-scale switch have no test or fixture in the reference
-(kernel_test.py:58 leaves them as a TODO): they are restated from the source
-text alone and are therefore "parity unpinned" beyond the closed forms checked
-in tests/test_oracle.py.
+(kernel_test.py:58 leaves them as a TODO): they are pinned by tables of fp16
+bit patterns typed by hand from the reference's text (every code of every bit
+width, the added zero, the negated scale, the single rounding, -0.0 and NaN
+scales) in tests/test_oracle.py.
 
 Dimension names: K = reduction dim (unpacked weight rows), S = output columns,
 R = packed rows, g = group size.
@@ -173,7 +174,8 @@ def sparse_unpack(matrix: np.ndarray, mask: np.ndarray):
 # pinned by (linear): IEEE-754: numpy float16 subtract and multiply are each
 # correctly rounded, as __hsub/__hmul are; checked exhaustively against an
 # independent float64-then-round evaluation in tests.  Exponent mode: closed
-# form in float64 rounded once (a power of two times s is exact); source-only.
+# form in float64 rounded once (a power of two times s is exact); checked against
+# hand-typed fp16 bit patterns for every code of every bit width in tests.
 # --------------------------------------------------------------------------
 def dequant_linear(codes, scale, zero):
     """fp16( fp16( fp16(q) - z ) * s )  -- matmul.cuh:117-121."""

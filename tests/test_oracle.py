@@ -212,25 +212,67 @@ def test_dequant_linear_is_two_correctly_rounded_ops_exhaustive():
         assert OC.dequant_scalar(qi, 4, ss, zz).view(np.uint16) == step2.view(np.uint16)
 
 
+# Exponent quantisation, pinned by literal tables typed from the reference's text
+# (matmul.cuh:127-136: iv = (v & SGN ? -1 : 1) * (1 << (v & EXP_MSK)), SGN = 1 << (bits - 1),
+# EXP_MSK = SGN - 1, result = __hfma(half(iv), scale, zero); matmul.cuh:414-428: a stored scale
+# below zero selects this branch and is negated first).  Every entry is an fp16 bit pattern worked
+# out by hand; nothing here evaluates the oracle's own expression.
+#   stored scale -0.5 (0xB800), zero 3.0 (0x4200): w = 3 + 0.5 * iv
+EXPO_TABLE = {
+    # iv:   +1      +2      +4      +8      +16     +32     +64     +128    -1      -2      -4      -8      -16     -32     -64     -128
+    4: [0x4300, 0x4400, 0x4500, 0x4700, 0x4980, 0x4CC0, 0x5060, 0x5430, 0x4100, 0x4000, 0x3C00, 0xBC00, 0xC500, 0xCA80, 0xCF40, 0xD3A0],
+    # iv:   +1      +2      +4      +8      -1      -2      -4      -8
+    3: [0x4300, 0x4400, 0x4500, 0x4700, 0x4100, 0x4000, 0x3C00, 0xBC00],
+    # iv:   +1      +2      -1      -2
+    2: [0x4300, 0x4400, 0x4100, 0x4000],
+}
+#   int3, stored scale -0.75 (0xBA00), zero -1.25 (0xBD00): w = -1.25 + 0.75 * iv
+#   = -0.5, 0.25, 1.75, 4.75, -2, -2.75, -4.25, -7.25
+EXPO_TABLE_INT3_B = [0xB800, 0x3400, 0x3F00, 0x44C0, 0xC000, 0xC180, 0xC440, 0xC740]
+
+
+def _h(bits16):
+    return np.array(bits16, dtype=np.uint16).view(np.float16)
+
+
 @pytest.mark.parametrize("bits", [4, 3, 2])
-def test_dequant_exponent_closed_forms(bits):
-    half = 1 << (bits - 1)
-    for v in range(1 << bits):
-        e = v & (half - 1)
-        sign = -1.0 if v & half else 1.0
-        # unit scale, zero offset: exactly +-2^e
-        assert float(O.dequant_exponent(bits, v, np.float16(1), np.float16(0))) == sign * 2.0 ** e
-        # stored scale negative selects the branch and is negated (matmul.cuh:424-427)
-        got = O.dequant_dynamic(bits, v, np.float16(-0.5), np.float16(3.0))
-        assert float(got) == 3.0 + sign * 0.5 * 2.0 ** e
-        assert float(OC.dequant_scalar(v, bits, np.float16(-0.5), np.float16(3.0))) == float(got)
-    # single rounding of the fused multiply-add: 1 * 0.1h + 2048 rounds once
-    s, z = np.float16(0.0999755859375), np.float16(2048)
-    exact = Fraction(float(s)) + Fraction(2048)
-    assert O.dequant_exponent(4, 0, s, z).view(np.uint16) == _round_half(exact).view(np.uint16)
-    # scale >= 0 keeps the linear branch; -0.0 counts as >= 0
-    assert float(O.dequant_dynamic(4, 5, np.float16(-0.0), np.float16(1.0))) == 0.0
-    assert float(O.dequant_dynamic(4, 5, np.float16(2.0), np.float16(1.0))) == 8.0
+def test_dequant_exponent_literal_table(bits):
+    scale, zero = _h(0xB800), _h(0x4200)                  # -0.5, 3.0
+    for v, want in enumerate(EXPO_TABLE[bits]):
+        got = O.dequant_dynamic(bits, v, scale, zero)
+        assert int(np.asarray(got).view(np.uint16)) == want, (bits, v)
+        assert int(OC.dequant_scalar(v, bits, scale, zero).view(np.uint16)) == want, (bits, v)
+        # the stand-alone exponent routine takes the already negated scale
+        assert int(np.asarray(O.dequant_exponent(bits, v, _h(0x3800), zero)).view(np.uint16)) == want
+    # bits above the field are ignored (the decoders hand over unmasked shifted words, matmul.cuh:131-134)
+    assert int(np.asarray(O.dequant_dynamic(bits, (1 << bits) | 1, scale, zero)).view(np.uint16)) == EXPO_TABLE[bits][1]
+
+
+def test_dequant_exponent_literal_table_int3_second_scale():
+    scale, zero = _h(0xBA00), _h(0xBD00)                  # -0.75, -1.25
+    for v, want in enumerate(EXPO_TABLE_INT3_B):
+        assert int(np.asarray(O.dequant_dynamic(3, v, scale, zero)).view(np.uint16)) == want, v
+        assert int(OC.dequant_scalar(v, 3, scale, zero).view(np.uint16)) == want, v
+
+
+def test_dequant_exponent_is_one_fused_rounding_and_the_switch():
+    # zero is ADDED (not subtracted) and the multiply-add rounds once:
+    #   code 3 (iv = +8), stored scale -0.0999755859375 (0xAE66), zero 1000 (0x63D0):
+    #   1000 + 0.7998046875 = 1000.7998..., fp16 spacing there is 0.5 -> 1001.0 = 0x63D2
+    assert int(np.asarray(O.dequant_dynamic(4, 3, _h(0xAE66), _h(0x63D0))).view(np.uint16)) == 0x63D2
+    assert int(OC.dequant_scalar(3, 4, _h(0xAE66), _h(0x63D0)).view(np.uint16)) == 0x63D2
+    # no intermediate overflow: code 7 (iv = +128), stored scale -600 (0xE0B0), zero -60000 (0xFB53):
+    # 76800 - 60000 = 16800 = 0x741A, although 76800 alone is beyond fp16 (a separate multiply gives inf)
+    assert int(np.asarray(O.dequant_dynamic(4, 7, _h(0xE0B0), _h(0xFB53))).view(np.uint16)) == 0x741A
+    assert int(OC.dequant_scalar(7, 4, _h(0xE0B0), _h(0xFB53)).view(np.uint16)) == 0x741A
+    # the switch is `scale >= 0` (matmul.cuh:420): -0.0 stays linear: (5 - 1) * -0.0 = -0.0 = 0x8000;
+    # +2.0 is linear: (5 - 1) * 2 = 8 = 0x4800; a NaN scale fails the comparison and takes the
+    # exponent branch, whose result is NaN
+    assert int(np.asarray(O.dequant_dynamic(4, 5, _h(0x8000), _h(0x3C00))).view(np.uint16)) == 0x8000
+    assert int(OC.dequant_scalar(5, 4, _h(0x8000), _h(0x3C00)).view(np.uint16)) == 0x8000
+    assert int(np.asarray(O.dequant_dynamic(4, 5, _h(0x4000), _h(0x3C00))).view(np.uint16)) == 0x4800
+    assert np.isnan(float(O.dequant_dynamic(4, 5, _h(0x7E00), _h(0x3C00))))
+    assert np.isnan(float(OC.dequant_scalar(5, 4, _h(0x7E00), _h(0x3C00))))
 
 
 @pytest.mark.parametrize("bits,sparse", [(4, False), (3, False), (2, False), (4, True)])
