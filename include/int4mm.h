@@ -57,6 +57,7 @@ extern "C" {
 #define INT4MM_ERR_WORKSPACE    6   /* workspace missing or smaller than int4mm_workspace_bytes()    */
 #define INT4MM_ERR_LAUNCH       7   /* the HIP runtime refused the launch; see int4mm_last_hip_error */
 #define INT4MM_ERR_ALIGN        8   /* a pointer is not 16-byte aligned                              */
+#define INT4MM_ERR_HANDOVER     9   /* a matvec hand-over timed out on this workspace (see int4mm_workspace_status) */
 
 /* Human-readable text for a code above (host pointer, static storage). */
 INT4MM_API const char* int4mm_error_string(int code);
@@ -66,7 +67,7 @@ INT4MM_API int int4mm_last_hip_error(void);
 INT4MM_API int int4mm_abi_version(void);
 
 /* Benchmark / tuning hook, not part of the drop-in boundary: overrides a launch
- * heuristic process-wide (value 0 restores the default).  key 0 = waves per
+ * heuristic for the calling host thread (value 0 restores the default).  key 0 = waves per
  * workgroup of the matvec and few-row kernels, 1 = matvec 64-row units per lane
  * group, 2 = matvec lane groups per wave (1, 2, 4), 3 = matmul kernel variant
  * (5 / 6 / 7 = pipelined 256x128 / 256x256 / 128x256 tiles, 9 = 256x256 without
@@ -77,7 +78,8 @@ INT4MM_API int int4mm_abi_version(void);
  * filled round are not split, 8 = the few-row kernel whose waves share the
  * staged states: 1 = never, n >= 2 = from n rows on whatever the shape,
  * 9 = address of a device buffer of int64 [workgroups][8][16]: the dense int4 matvec then runs
- * its instrumented variant and records time stamps there (see matvec_timeline.py). */
+ * its instrumented variant and records time stamps there (see matvec_timeline.py),
+ * 10 = polls after which a matvec hand-over gives up (failure-handling tests). */
 INT4MM_API int int4mm_tune(int key, int64_t value);
 
 /* Shape of one product.  matrix_rows = R, n_groups = G (rows of scales/zeros).
@@ -107,6 +109,22 @@ typedef struct int4mm_shape {
  * for partial tiles), so always pass the size the buffer was zero-filled with. */
 INT4MM_API size_t int4mm_workspace_bytes(int64_t max_out_size);
 INT4MM_API int int4mm_workspace_init(void* workspace, size_t workspace_bytes, void* stream);
+
+/* Health of a workspace.  The matvec's workgroups hand partial sums over through the workspace;
+ * the last workgroup of a column range waits for the others with a bounded number of polls.  If
+ * that wait ever runs out (it cannot while the GPU dispatches workgroups in order), the affected
+ * outputs are NaN, the workspace is marked, and every later matvec on it returns NaN too -- never a
+ * silently wrong number -- until int4mm_workspace_init has zero-filled it again.  This call copies
+ * the mark back on `stream`, waits for it and returns INT4MM_ERR_HANDOVER if it is set.  No
+ * counterpart in the reference, whose atomics cannot time out (matvec_kernel.cu:263). */
+INT4MM_API int int4mm_workspace_status(void* workspace, size_t workspace_bytes, void* stream);
+
+/* Which kernel, tile shape and split would int4mm_matvec (product 0) or int4mm_matmul (product 1)
+ * launch for `shape` with a workspace of `workspace_bytes`?  Writes a one-line description into
+ * `text` (host memory) using the launcher's own decision code with the launches switched off; it
+ * touches no GPU.  For tests that pin the dispatch of the benchmark shapes, and for profiling. */
+INT4MM_API int int4mm_describe_launch(int product, int bits, const int4mm_shape* shape, int sparse,
+                  size_t workspace_bytes, char* text, size_t text_bytes);
 
 /* Bytes of workspace with which int4mm_matmul may split the K dimension of `shape`
  * over several workgroups per output tile (shapes with so few tiles that most of

@@ -15,7 +15,7 @@ LIB_NAME = "libint4mm_hip.so"
 EXPORTS = [
     "int4mm_error_string", "int4mm_last_hip_error", "int4mm_abi_version", "int4mm_tune",
     "int4mm_workspace_bytes", "int4mm_workspace_init", "int4mm_matmul_workspace_bytes", "int4mm_matvec", "int4mm_matmul",
-    "int4mm_matvec_static",
+    "int4mm_matvec_static", "int4mm_workspace_status", "int4mm_describe_launch",
     "int4mm_sparse_pack", "int4mm_dense_pack", "int4mm_unpack", "int4mm_dequantize",
 ]
 
@@ -64,6 +64,10 @@ def lib():
         f.argtypes = [C.c_int, vp, vp, vp, vp, vp, vp, C.POINTER(Shape), vp, sz, vp]
     L.int4mm_matvec_static.restype = C.c_int
     L.int4mm_matvec_static.argtypes = [C.c_int, vp, vp, vp, vp, vp, vp, C.POINTER(Shape), vp]
+    L.int4mm_workspace_status.restype = C.c_int
+    L.int4mm_workspace_status.argtypes = [vp, sz, vp]
+    L.int4mm_describe_launch.restype = C.c_int
+    L.int4mm_describe_launch.argtypes = [C.c_int, C.c_int, C.POINTER(Shape), C.c_int, sz, C.c_char_p, sz]
     L.int4mm_sparse_pack.restype = C.c_int
     L.int4mm_sparse_pack.argtypes = [vp, vp, vp, vp, i64, i64, vp, vp]
     L.int4mm_dense_pack.restype = C.c_int
@@ -92,6 +96,24 @@ def _check(rc, what):
 
 def tune(key: int, value: int):
     _check(lib().int4mm_tune(key, value), "int4mm_tune")
+
+
+def describe_launch(product, bits, batch, seq_len, in_size, out_size, group_size=128, sparse=False, workspace_bytes=None):
+    """one line saying which kernel / tile shape / split ``matvec`` ("vec") or ``matmul`` ("mtx") would launch"""
+    rows = in_size // 16 if sparse else in_size * bits // 32
+    groups = 1 if group_size < 0 else -(-in_size // group_size)
+    sh = Shape(batch, seq_len, in_size, out_size, rows, groups, group_size)
+    if workspace_bytes is None:
+        workspace_bytes = lib().int4mm_matmul_workspace_bytes(C.byref(sh), 1 if sparse else 0)
+    buf = C.create_string_buffer(512)
+    _check(lib().int4mm_describe_launch(0 if product == "vec" else 1, bits, C.byref(sh), 1 if sparse else 0,
+                                        workspace_bytes, buf, 512), "int4mm_describe_launch")
+    return buf.value.decode()
+
+
+def workspace_status(workspace):
+    """0 if healthy; raises Int4mmError(code 9) after a matvec hand-over timed out on it"""
+    _check(lib().int4mm_workspace_status(_ptr(workspace), workspace.numel(), _stream()), "int4mm_workspace_status")
 
 
 def new_workspace(out_size: int, device="cuda"):

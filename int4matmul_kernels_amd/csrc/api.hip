@@ -3,13 +3,33 @@
 #include "common.h"
 
 #include <atomic>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
 
 namespace i4 {
 
 static thread_local int g_last_hip_error = 0;
-static std::atomic<int64_t> g_tuning[TUNE_COUNT];
+static thread_local int64_t g_tuning[TUNE_COUNT];
+static thread_local bool g_noting = false;
+static thread_local char g_note[512];
+
+bool is_noting() { return g_noting; }
+bool noting(const char* fmt, ...) {
+    if (!g_noting) return false;
+    const size_t used = strlen(g_note);
+    if (used + 2 < sizeof(g_note)) {
+        va_list ap;
+        va_start(ap, fmt);
+        vsnprintf(g_note + used, sizeof(g_note) - used, fmt, ap);
+        va_end(ap);
+        strncat(g_note, "; ", sizeof(g_note) - strlen(g_note) - 1);
+    }
+    return true;
+}
 
 int check_launch(const char*) {
+    if (g_noting) return INT4MM_OK;
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) {
         g_last_hip_error = (int)e;
@@ -18,7 +38,7 @@ int check_launch(const char*) {
     return INT4MM_OK;
 }
 
-int64_t tuning(int key) { return (key >= 0 && key < TUNE_COUNT) ? g_tuning[key].load() : 0; }
+int64_t tuning(int key) { return (key >= 0 && key < TUNE_COUNT) ? g_tuning[key] : 0; }
 
 static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
@@ -76,6 +96,7 @@ const char* int4mm_error_string(int code) {
         case INT4MM_ERR_WORKSPACE: return "workspace missing or too small";
         case INT4MM_ERR_LAUNCH: return "HIP launch failed";
         case INT4MM_ERR_ALIGN: return "a device pointer is not 16-byte aligned";
+        case INT4MM_ERR_HANDOVER: return "a matvec hand-over timed out earlier on this workspace; zero-fill it again";
         default: return "unknown int4mm error";
     }
 }
@@ -83,16 +104,17 @@ const char* int4mm_error_string(int code) {
 int int4mm_last_hip_error(void) { return g_last_hip_error; }
 int int4mm_abi_version(void) { return 1; }
 
-// Benchmark/tuning hook: overrides a launch heuristic (0 restores the default).
+// Benchmark/tuning hook: overrides a launch heuristic for the calling thread (0 restores the default).
 // Keys: 0 = matvec waves per workgroup, 1 = matvec units per lane group,
 // 2 = matvec lane groups per wave (1, 2 or 4), 3 = matmul kernel variant,
 // 4 = matvec: 1 disables the software prefetch, 5 = 1 disables the few-row kernel,
 // 6 = matmul split-K factor (1 = never, 2..8 = forced where the shape allows a split),
 // 7 = 1: the tiles of a matmul's last, partly filled round are not split,
-// 8 = 1: 33 .. 96 rows take the few-row kernel whose waves stage their own states.
+// 8 = 1: 33 .. 96 rows take the few-row kernel whose waves stage their own states,
+// 9 = address of the matvec's time-stamp buffer, 10 = polls before a matvec hand-over gives up.
 int int4mm_tune(int key, int64_t value) {
     if (key < 0 || key >= TUNE_COUNT) return INT4MM_ERR_SHAPE;
-    g_tuning[key].store(value);
+    g_tuning[key] = value;
     return INT4MM_OK;
 }
 
@@ -108,6 +130,38 @@ int int4mm_workspace_init(void* workspace, size_t workspace_bytes, void* stream)
     hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
                        (hipStream_t)stream, (uint32_t*)workspace, n);
     return check_launch("workspace_init");
+}
+
+
+// What would int4mm_matvec (product 0) or int4mm_matmul (product 1) launch for this shape?  Runs the
+// launcher's own decision code with the launches switched off; needs no GPU.
+int int4mm_describe_launch(int product, int bits, const int4mm_shape* shape, int sparse, size_t workspace_bytes,
+                           char* text, size_t text_bytes) {
+    if (shape == nullptr || text == nullptr || text_bytes == 0) return INT4MM_ERR_NULL;
+    void* fake = reinterpret_cast<void*>(uintptr_t(1) << 20);          // aligned, never dereferenced on the host
+    g_note[0] = 0;
+    g_noting = true;
+    const int rc = (product == 0 ? int4mm_matvec : int4mm_matmul)(bits, fake, fake, fake, fake, fake, sparse ? fake : nullptr, shape,
+                                                                  workspace_bytes ? fake : nullptr, workspace_bytes, nullptr);
+    g_noting = false;
+    snprintf(text, text_bytes, "%s", g_note);
+    return rc;
+}
+
+// Has a matvec hand-over on this workspace timed out since it was last zero-filled?  (Copies one word
+// back on `stream` and waits for it.)  After INT4MM_ERR_HANDOVER every matvec on the workspace returns
+// NaN until int4mm_workspace_init has run again.
+int int4mm_workspace_status(void* workspace, size_t workspace_bytes, void* stream) {
+    if (workspace == nullptr) return INT4MM_ERR_NULL;
+    const WorkspaceParts p = workspace_parts(workspace, workspace_bytes);
+    if (p.counters == nullptr) return INT4MM_ERR_WORKSPACE;
+    uint32_t word = 0;
+    if (hipMemcpyAsync(&word, p.counters - 8, 4, hipMemcpyDeviceToHost, (hipStream_t)stream) != hipSuccess ||
+        hipStreamSynchronize((hipStream_t)stream) != hipSuccess) {
+        g_last_hip_error = (int)hipGetLastError();
+        return INT4MM_ERR_LAUNCH;
+    }
+    return word ? INT4MM_ERR_HANDOVER : INT4MM_OK;
 }
 
 }  // extern "C"

@@ -87,9 +87,15 @@ int check_launch(const char* what);           // returns INT4MM_OK or INT4MM_ERR
 int validate_product(int bits, const void* outs, const void* matrix, const void* multiplier,
                      const void* scales, const void* zeros, const void* sparse_mask,
                      const int4mm_shape* sh, bool matvec);
-int64_t tuning(int key);                       // see int4mm_tune
+int64_t tuning(int key);                       // see int4mm_tune (values are per host thread)
 enum TuneKey { TUNE_MV_WAVES = 0, TUNE_MV_UNITS = 1, TUNE_MV_LK = 2, TUNE_MM_VARIANT = 3, TUNE_MV_NOPF = 4,
-               TUNE_NO_SKINNY = 5, TUNE_MM_SPLIT = 6, TUNE_MM_TAIL = 7, TUNE_NO_WIDE = 8, TUNE_MV_TIMELINE = 9, TUNE_COUNT = 10 };
+               TUNE_NO_SKINNY = 5, TUNE_MM_SPLIT = 6, TUNE_MM_TAIL = 7, TUNE_NO_WIDE = 8, TUNE_MV_TIMELINE = 9,
+               TUNE_MV_SPIN = 10, TUNE_COUNT = 11 };
+
+// int4mm_describe_launch: while this thread is "noting", a launcher records the kernel and launch
+// shape it has chosen instead of launching it.  noting(...) returns true (skip the launch) in that mode.
+bool noting(const char* fmt, ...) __attribute__((format(printf, 1, 2)));
+bool is_noting();
 
 // few-row product (2 .. 96 rows; sparse_mask != nullptr: 16:32 int4); false = shape not taken, use the general kernels
 bool skinny_rows(int bits, _Float16* outs, const uint32_t* matrix, const _Float16* x, const _Float16* scales,
@@ -105,7 +111,8 @@ size_t skinny_workspace_bytes(int64_t R, int64_t K, int64_t S, bool sparse);
 // hand-over slots from byte 0 and, in its last page, the arrival counters of the split-K kernels.  The
 // upper half is scratch for partial tiles; no call relies on what it holds.
 struct WorkspaceParts {
-    char* counters;           // one page (nullptr: the workspace has no room for it)
+    char* counters;           // one page (nullptr: the workspace has no room for it); the 8 bytes in front of it
+                              // are the matvec's hand-over error word (non-zero: a hand-over timed out)
     char* scratch;
     size_t slots_bytes;       // room for the matvec's slots, below the counters
     size_t scratch_bytes;

@@ -899,6 +899,9 @@ static void launch_pipe(MatmulArgs a, int64_t B, hipStream_t st) {
     const int total = a.tiles_m * a.tiles_n;
     const dim3 grid(a.split_from + (total - a.split_from) * a.ksplit, 1, (unsigned)B), block(NW * 128);
     a.by_columns = a.tiles_n % 8 == 0;
+    if (noting("matmul_kernel_pipe<bits=%d,%s,tile=%dx%d,%s> tiles=%d ksplit=%d split_from=%d workgroups=%u batch=%d", BITS,
+               SPARSE ? "16:32" : "dense", TM * 64, NW * 64, PING ? "two-phase" : "plain", total, a.ksplit, a.split_from, grid.x, (int)B))
+        return;
     if (a.ksplit > 1) {
         hipLaunchKernelGGL((matmul_kernel_pipe<BITS, SPARSE, NW, TM, PING, true>), grid, block, 0, st, a);
         return;
@@ -952,6 +955,7 @@ static void launch_tile(MatmulArgs a, int64_t B, hipStream_t st) {
     a.tiles_m = (a.M + BM - 1) / BM;
     a.tiles_n = (a.S + BN - 1) / BN;
     const dim3 grid(a.tiles_m * a.tiles_n, 1, (unsigned)B), block((BM / WM) * (BN / WN) * 64);
+    if (noting("matmul_kernel<bits=%d,%s,tile=%dx%d> tiles=%u batch=%d", BITS, SPARSE ? "16:32" : "dense", BM, BN, grid.x, (int)B)) return;
     hipLaunchKernelGGL((matmul_kernel<BITS, SPARSE, BM, BN, WM, WN>), grid, block, 0, st, a);
 }
 

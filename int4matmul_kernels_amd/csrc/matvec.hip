@@ -52,6 +52,8 @@ struct MatvecArgs {
     int units_per_wg;
     int group_units;        // group size in units (>= 1); huge for a single group
     int splits;             // == gridDim.y
+    uint32_t* sticky;       // hand-over error word of the workspace (non-zero: poisoned)
+    int spin_limit;         // polls before a reader gives up
     uint64_t* timeline;     // instrumented variant only: 16 time stamps per wave (8 wave slots per workgroup)
 };
 
@@ -688,9 +690,12 @@ void matvec_kernel(MatvecArgs a) {
         stamp(13); stamp(15);
         return;
     }
+    // (a hand-over that timed out earlier may have left late slots behind: the workspace stays
+    // poisoned -- every result NaN -- until the host zero-fills it again)
+    const uint32_t poisoned = __hip_atomic_load(a.sticky, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     for_owned([&](int i, int ocol) {
         float sum = (float)a.outs[ocol];
-        bool ok = true;
+        bool ok = poisoned == 0;
         // slots are fetched eight at a time so that their latencies overlap; a
         // slot that is not full yet is polled again on its own
         for (int s0 = 0; s0 < a.splits - 1; s0 += 8) {
@@ -703,7 +708,7 @@ void matvec_kernel(MatvecArgs a) {
                 if (s0 + k >= a.splits - 1) break;
                 uint64_t* p = &a.slots[(int64_t)(s0 + k) * a.S + ocol];
                 int spins = 0;
-                while ((uint32_t)(v[k] >> 32) != SLOT_FULL && spins < MV_SPIN_LIMIT) {
+                while ((uint32_t)(v[k] >> 32) != SLOT_FULL && spins < a.spin_limit) {
                     __builtin_amdgcn_s_sleep(1);
                     v[k] = slot_load(p);
                     ++spins;
@@ -714,8 +719,10 @@ void matvec_kernel(MatvecArgs a) {
             }
         }
         sum += total[i];
-        // a slot that never arrived (which would mean a writer was never run)
-        // poisons the output instead of hanging the wave
+        // a slot that never arrived (which would mean a writer was never run) poisons the
+        // output -- and the workspace, since the writer may still fill its slot later --
+        // instead of hanging the wave
+        if (!ok) __hip_atomic_store(a.sticky, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         a.outs[ocol] = ok ? (h16)sum : (h16)__builtin_nanf("");
     });
     stamp(13); stamp(15);
@@ -806,9 +813,14 @@ static int matvec_impl(int bits, void* outs, const void* matrix, const void* mul
     a.group_units = (int)(g / 64 > 0x7FFFFFF ? 0x7FFFFFF : g / 64);
     a.splits = splits;
     a.timeline = (uint64_t*)(uintptr_t)tuning(TUNE_MV_TIMELINE);
+    a.sticky = splits > 1 ? reinterpret_cast<uint32_t*>(workspace_parts(workspace, workspace_bytes).counters - 8) : nullptr;
+    a.spin_limit = tuning(TUNE_MV_SPIN) > 0 ? (int)tuning(TUNE_MV_SPIN) : MV_SPIN_LIMIT;
 
     const dim3 grid(strips, splits, 1), block(waves * WAVE);
     hipStream_t st = (hipStream_t)stream;
+    if (noting("matvec_kernel<bits=%d,%s,lane_groups=%d,prefetch=%d> strips=%d splits=%d waves=%d units_per_workgroup=%d batch=%d",
+               bits, sparse_mask ? "16:32" : "dense", lk, (int)pf, strips, splits, waves, upwg, (int)B))
+        return INT4MM_OK;
     for (int64_t b = 0; b < B; ++b) {                      // one pass over the weights per batch row
         a.outs = (h16*)outs + b * S;
         a.x = (const h16*)multiplier + b * K;

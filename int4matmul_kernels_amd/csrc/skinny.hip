@@ -924,6 +924,9 @@ static bool launch_wide(SkinnyArgs a, const WidePlan& p, hipStream_t st) {
     a.block_rows = p.block_rows;
     a.units_per_split = p.units_per_split;
     const dim3 grid((unsigned)(a.S / 256), (unsigned)p.row_blocks, (unsigned)p.ksplit), block(512);
+    if (noting("wide_rows_kernel<bits=%d,%s,row_tiles=%d> strips=%u row_blocks=%u ksplit=%u", BITS, SPARSE ? "16:32" : "dense", p.mt,
+               grid.x, grid.y, grid.z))
+        return true;
     auto go = [&](auto kernel, int slot) {
         static std::atomic<uint64_t> done[4];
         int dev = 0;
@@ -953,6 +956,9 @@ static bool launch_skinny(const SkinnyArgs& a, int waves, int ksplit, hipStream_
     if (red > lds) lds = red;
     if (lds > 150 * 1024 - (SPARSE ? 4096 : 0)) return false;      // (16:32: 4 KB of static LDS for the selector table)
     const dim3 grid(strips, (a.R + 31) / 32, ksplit), block(waves * 64);
+    if (noting("skinny_kernel<bits=%d,%s,columns_per_lane=%d,row_tiles=%d> strips=%d row_blocks=%u ksplit=%d waves=%d", BITS,
+               SPARSE ? "16:32" : "dense", CW, rt <= 1 ? 1 : (rt <= 2 ? 2 : 4), strips, grid.y, ksplit, waves))
+        return true;
     auto go = [&](auto kernel, int slot) {
         // more than 64 KB of dynamic LDS has to be requested once per kernel and device
         static std::atomic<uint64_t> done[3];

@@ -28,7 +28,7 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(lib, n), f"{n} is declared in include/int4mm.h but not exported"
     assert sorted(capi.EXPORTS) == names
     assert lib.int4mm_abi_version() == 1
-    for code in range(0, 9):
+    for code in range(0, 10):
         assert lib.int4mm_error_string(code)
 
 

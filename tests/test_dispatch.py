@@ -1,0 +1,73 @@
+"""Host-only: which kernel, tile shape and split the launchers choose for every
+benchmark configuration.  ``int4mm_describe_launch`` runs the launchers' own
+decision code with the launches switched off, so an edit of a shape rule that
+silently reroutes one of these shapes fails here, without a GPU."""
+import pytest
+
+from int4matmul_kernels_amd import capi
+
+K, S = 5120, 20480
+
+
+def d(*a, **kw):
+    return capi.describe_launch(*a, **kw)
+
+
+def test_matvec_configurations():
+    # C1: K = S = 1024, g = 64
+    assert d("vec", 4, 1, 1, 1024, 1024, 64).startswith(
+        "matvec_kernel<bits=4,dense,lane_groups=4,prefetch=0> strips=16 splits=4 waves=1 units_per_workgroup=4")
+    # C2 and its transposed shape: 640 workgroups of four waves
+    assert d("vec", 4, 1, 1, K, S, 128).startswith(
+        "matvec_kernel<bits=4,dense,lane_groups=2,prefetch=0> strips=160 splits=4 waves=4 units_per_workgroup=20")
+    assert d("vec", 4, 1, 1, S, K, 128).startswith(
+        "matvec_kernel<bits=4,dense,lane_groups=4,prefetch=0> strips=80 splits=8 waves=4 units_per_workgroup=40")
+    # C4: 16:32 at K = S = 16384, g = 64
+    assert d("vec", 4, 1, 1, 16384, 16384, 64, sparse=True).startswith(
+        "matvec_kernel<bits=4,16:32,lane_groups=4,prefetch=1> strips=256 splits=3 waves=4 units_per_workgroup=86")
+    # C5: int3 / int2 take the shape of C2
+    for bits in (3, 2):
+        assert d("vec", bits, 1, 1, K, S, 128).startswith(
+            f"matvec_kernel<bits={bits},dense,lane_groups=2,prefetch=0> strips=160 splits=4 waves=4 units_per_workgroup=20")
+
+
+@pytest.mark.parametrize("bits", [4, 3, 2])
+def test_dense_matmul_m2048(bits):
+    # 640 tiles of 256 x 256 in the two-phase order; the 128 tiles of the third round split in two along K
+    want = (f"matmul_kernel_pipe<bits={bits},dense,tile=256x256,two-phase> tiles=640 ksplit=2 split_from=512 "
+            "workgroups=768")
+    assert d("mtx", bits, 1, 2048, K, S, 128).startswith(want)
+    # without room for the partial tiles the last round stays whole
+    assert "ksplit=1 split_from=0 workgroups=640" in d("mtx", bits, 1, 2048, K, S, 128, workspace_bytes=0)
+
+
+def test_other_matmul_configurations():
+    assert d("mtx", 4, 1, 2048, S, K, 128).startswith("matmul_kernel_pipe<bits=4,dense,tile=256x256,two-phase> tiles=160")
+    # C3 small: one group, 16 tiles of the general kernel (the pipelined kernel's prologue would dominate)
+    assert d("mtx", 4, 1, 2048, 128, 128, 128).startswith("matmul_kernel<bits=4,dense,tile=128x128> tiles=16")
+    # C4: the 16:32 format keeps the plain order (its decode has no registers to spare)
+    assert d("mtx", 4, 1, 2048, K, S, 64, sparse=True).startswith(
+        "matmul_kernel_pipe<bits=4,16:32,tile=256x256,plain> tiles=640 ksplit=2 split_from=512 workgroups=768")
+
+
+def test_few_rows_and_batches():
+    assert d("mtx", 4, 1, 8, K, S, 128).startswith("skinny_kernel<bits=4,dense,columns_per_lane=4,row_tiles=1> strips=320")
+    assert d("vec", 4, 8, 1, K, S, 128).startswith("skinny_kernel<bits=4,dense,columns_per_lane=4,row_tiles=1> strips=320")
+    assert d("mtx", 4, 1, 64, K, S, 128).startswith("wide_rows_kernel<bits=4,dense,row_tiles=4> strips=80 row_blocks=1 ksplit=3")
+    assert d("mtx", 4, 1, 16, S, K, 128).startswith("skinny_kernel<bits=4,dense")
+    assert d("mtx", 4, 1, 257, K, S, 128).startswith("matmul_kernel_pipe<bits=4,dense,tile=128x256")
+
+
+def test_tuning_is_per_thread_and_describe_leaves_no_trace():
+    import threading
+    capi.tune(3, 1)
+    try:
+        seen = {}
+        t = threading.Thread(target=lambda: seen.setdefault("other", d("mtx", 4, 1, 2048, K, S, 128)))
+        t.start()
+        t.join()
+        assert seen["other"].startswith("matmul_kernel_pipe")            # the other thread keeps the defaults
+        assert d("mtx", 4, 1, 2048, K, S, 128).startswith("matmul_kernel<bits=4,dense,tile=128x128>")
+    finally:
+        capi.tune(3, 0)
+    assert d("mtx", 4, 1, 2048, K, S, 128).startswith("matmul_kernel_pipe")
