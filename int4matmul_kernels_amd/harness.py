@@ -4,7 +4,8 @@ Plays the role of the reference's `kernel_test.py` (generation of test
 matrices `:160-236`, call convention `:254-259`, error metric `:261-262`, pass
 rule `:344-348`, timing loop `:290-309`, markdown table `:359-391`) through the
 drop-in `int4matmul` extension module, with three differences: matrices are
-packed on the device by the library's own packers, each row also reports the
+packed on the device by the library's own packers (the expected values come from
+the unpacked codes, in plain torch arithmetic), each row also reports the
 roofline figure of the kernel (GB/s for M = 1, TFLOP/s otherwise), and launches
 are additionally timed with HIP events.
 
@@ -77,23 +78,26 @@ def make_case(bits, K, S, M, group, sparse, B, seed=0):
     else:
         matrix = torch.zeros((K * bits // 32, S), dtype=torch.int32, device=DEV)
         capi.dense_pack(bits, matrix, codes_d)
+    keep_ks = keep_d.t().contiguous() if sparse else None            # [K, S], 1 = kept
     return dict(bits=bits, K=K, S=S, M=M, B=B, group=group, matrix=matrix, mask=mask,
-                scales=scales.to(DEV), zeros=zeros.to(DEV), states=states.to(DEV))
+                scales=scales.to(DEV), zeros=zeros.to(DEV), states=states.to(DEV), codes=codes_d, keep=keep_ks)
 
 
 def reference_matrices(c):
-    """(fp16 weights exactly as the kernels' decode defines them, fp32 weights
-    dequantised in fp32) -- both through the library's unpack, then torch math"""
-    K, S, bits = c["K"], c["S"], c["bits"]
-    w16 = torch.empty((K, S), dtype=torch.float16, device=DEV)
-    capi.dequantize(bits, w16, c["matrix"], c["scales"], c["zeros"], c["group"], c["mask"])
-    codes = torch.empty((K, S), dtype=torch.uint8, device=DEV)
-    keep = torch.empty((K, S), dtype=torch.uint8, device=DEV)
-    capi.unpack(bits, codes, keep, c["matrix"], c["mask"])
+    """(fp16 weights as the reference's decode defines them, fp32 weights dequantised in fp32),
+    both from the UNPACKED codes and mask the case was generated with, in plain torch arithmetic
+    (kernel_test.py:138-157) -- nothing of the library's pack, unpack or dequantise is involved, so
+    a packing or decoding bug that the product kernels shared with the helpers would fail the gate"""
+    K = c["K"]
     g = K if c["group"] < 0 else c["group"]
     rows = torch.arange(K, device=DEV) // g
-    s32, z32 = c["scales"].float()[rows], c["zeros"].float()[rows]
-    w32 = (codes.float() - z32) * s32 * keep.float()
+    q = c["codes"]
+    s16, z16 = c["scales"][rows], c["zeros"][rows]
+    w16 = (q.half() - z16) * s16                                     # two fp16 roundings
+    w32 = (q.float() - z16.float()) * s16.float()
+    if c["keep"] is not None:
+        w16 = w16 * c["keep"].half()
+        w32 = w32 * c["keep"].float()
     return w16, w32
 
 
@@ -109,7 +113,7 @@ def algorithmic_bytes(c):
     return n
 
 
-def run_case(name, c, ext, repeats=100, trials=5):
+def run_case(name, c, ext, repeats=100, trials=5, cold=False):
     B, M, K, S = c["B"], c["M"], c["K"], c["S"]
     w16, w32 = reference_matrices(c)
     truth = c["states"].float() @ w32
@@ -138,10 +142,20 @@ def run_case(name, c, ext, repeats=100, trials=5):
             torch.cuda.synchronize()
             walls.append((time.time() - t0) / repeats)
         out[label + "_wall_us"] = sum(walls) / len(walls) * 1e6
-    # kernel-only: HIP events around back-to-back launches into one output buffer
+    # kernel-only: HIP events around back-to-back launches into one output buffer.  `cold`: the
+    # matvec rotates over enough copies of its weights (about 400 MB, more than the 256 MB
+    # last-level cache) that every launch streams them from HBM
     outs = torch.zeros((B, M, S), dtype=torch.float16, device=DEV)
-    call = lambda: ext.quant_matmul(c["bits"], outs, c["matrix"], c["states"], c["scales"], c["zeros"],
-                                    c["group"], c["mask"])
+    copies = [(c["matrix"], c["scales"], c["zeros"], c["mask"])]
+    if cold and M * B == 1:
+        while len(copies) * algorithmic_bytes(c) < 400e6:
+            copies.append(tuple(None if t is None else t.clone() for t in copies[0]))
+    state = {"i": 0}
+
+    def call():
+        m, sc, ze, mk = copies[state["i"] % len(copies)]
+        state["i"] += 1
+        ext.quant_matmul(c["bits"], outs, m, c["states"], sc, ze, c["group"], mk)
     n = 200 if M == 1 else 20
     for _ in range(5):
         call()
@@ -186,11 +200,15 @@ def main(argv=None):
     ap.add_argument("--quick", action="store_true", help="small shapes only")
     ap.add_argument("--config", action="append", default=[], help="bits,K,S,M,group,sparse[,B]")
     ap.add_argument("--repeats", type=int, default=100)
+    ap.add_argument("--cold", action="store_true", help="M = 1: rotate over copies of the weights so that every launch reads HBM")
+    ap.add_argument("--only", default="", help="comma-separated names of standard configurations to run")
     args = ap.parse_args(argv)
     if not torch.cuda.is_available():
         raise SystemExit("the harness needs a GPU")
     ext = pkg.load_extension()
     cases = QUICK if args.quick else STANDARD
+    if args.only:
+        cases = [c for c in STANDARD if c[0] in args.only.split(",")]
     if args.config:
         cases = []
         for i, spec in enumerate(args.config):
@@ -200,7 +218,7 @@ def main(argv=None):
     for case in cases:
         name, bits, K, S, M, group, sparse, B = case
         c = make_case(bits, K, S, M, group, sparse, B)
-        rows.append(run_case(name, c, ext, repeats=args.repeats))
+        rows.append(run_case(name, c, ext, repeats=args.repeats, cold=args.cold))
         print("%-5s int%d K=%d S=%d M=%d B=%d g=%d %s: %.2f us, %s, mean rel err %.2e %s" % (
             name, bits, K, S, M, B, group, "16:32" if sparse else "dense", rows[-1]["quant_event_us"],
             rows[-1]["rate"], rows[-1]["err_quant"], "ok" if rows[-1]["ok"] else "FAIL"), flush=True)

@@ -1,6 +1,6 @@
-"""The accuracy / timing harness runs its small configurations through the
-`int4matmul` extension and every case passes the reference's 10 % gate
-(kernel_test.py:344-348)."""
+"""The accuracy / timing harness runs through the `int4matmul` extension and every
+case passes the reference's 10 % gate (kernel_test.py:344-348): its small
+configurations, and one full-size benchmark configuration per format."""
 import pytest
 
 pytestmark = pytest.mark.gpu
@@ -15,3 +15,13 @@ def test_harness_quick_configurations():
         assert r["ok"], r
         assert r["err_quant"] < 0.1
         assert r["quant_event_us"] > 0
+
+
+def test_harness_full_size_row_per_format():
+    from int4matmul_kernels_amd import harness
+
+    names = ["C2", "C3", "C4v", "C5m3", "C5v2"]
+    rows = harness.main(["--only", ",".join(names), "--repeats", "2"])
+    assert [r["name"] for r in rows] == names
+    for r in rows:
+        assert r["ok"] and r["err_quant"] < 1e-2, r            # (mean relative error; the gate itself is 0.1)
