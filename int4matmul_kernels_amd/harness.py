@@ -12,6 +12,7 @@ are additionally timed with HIP events.
     python -m int4matmul_kernels_amd.harness                 # the standard configurations
     python -m int4matmul_kernels_amd.harness --quick         # small shapes only
     python -m int4matmul_kernels_amd.harness --config 4,5120,20480,2048,128,0
+    python -m int4matmul_kernels_amd.harness --only C3,C3t --clocks 3    # + shader clock under load
 
 A configuration is bits,K,S,M,group,sparse[,B].
 """
@@ -113,7 +114,47 @@ def algorithmic_bytes(c):
     return n
 
 
-def run_case(name, c, ext, repeats=100, trials=5, cold=False):
+def shader_clock_under_load(call, seconds):
+    """Median shader clock (MHz) that `rocm-smi --showclocks` reports while `call` is launched
+    back to back for `seconds`: what the GPU's power management leaves of its peak clock under
+    this kernel.  None when the tool gives no reading."""
+    import re
+    import subprocess
+    import threading
+
+    readings, stop = [], threading.Event()
+
+    def sample():
+        while not stop.is_set():
+            try:
+                text = subprocess.run(["rocm-smi", "--showclocks", "--csv"], capture_output=True, text=True,
+                                      timeout=5).stdout
+            except (OSError, subprocess.SubprocessError):
+                return
+            header = text.strip().splitlines()[0].split(",") if text.strip() else []
+            cols = [i for i, h in enumerate(header) if h.startswith("sclk clock speed")]
+            for line in text.strip().splitlines()[1:2]:
+                cells = line.split(",")
+                for i in cols:
+                    m = re.search(r"(\d+)Mhz", cells[i]) if i < len(cells) else None
+                    if m:
+                        readings.append(int(m.group(1)))
+            time.sleep(0.1)
+
+    th = threading.Thread(target=sample)
+    th.start()
+    t0 = time.time()
+    while time.time() - t0 < seconds:
+        for _ in range(20):
+            call()
+        torch.cuda.synchronize()
+    stop.set()
+    th.join()
+    readings = sorted(readings[1:])                       # the first one may predate the load
+    return readings[len(readings) // 2] if readings else None
+
+
+def run_case(name, c, ext, repeats=100, trials=5, cold=False, clocks=0.0):
     B, M, K, S = c["B"], c["M"], c["K"], c["S"]
     w16, w32 = reference_matrices(c)
     truth = c["states"].float() @ w32
@@ -175,6 +216,9 @@ def run_case(name, c, ext, repeats=100, trials=5, cold=False):
         out["rate"] = "%.0f GB/s" % (algorithmic_bytes(c) / us / 1e3)
     else:
         out["rate"] = "%.1f TFLOP/s" % (2.0 * B * M * K * S / us / 1e6)
+    if clocks > 0:
+        out["sclk_mhz"] = shader_clock_under_load(call, clocks)
+        out["fp16_sclk_mhz"] = shader_clock_under_load(fp16, clocks) if M > 1 else None
     return out
 
 
@@ -201,6 +245,8 @@ def main(argv=None):
     ap.add_argument("--config", action="append", default=[], help="bits,K,S,M,group,sparse[,B]")
     ap.add_argument("--repeats", type=int, default=100)
     ap.add_argument("--cold", action="store_true", help="M = 1: rotate over copies of the weights so that every launch reads HBM")
+    ap.add_argument("--clocks", type=float, default=0.0, metavar="SECONDS",
+                    help="also run each case for SECONDS and report the shader clock rocm-smi shows meanwhile")
     ap.add_argument("--only", default="", help="comma-separated names of standard configurations to run")
     args = ap.parse_args(argv)
     if not torch.cuda.is_available():
@@ -218,10 +264,12 @@ def main(argv=None):
     for case in cases:
         name, bits, K, S, M, group, sparse, B = case
         c = make_case(bits, K, S, M, group, sparse, B)
-        rows.append(run_case(name, c, ext, repeats=args.repeats, cold=args.cold))
-        print("%-5s int%d K=%d S=%d M=%d B=%d g=%d %s: %.2f us, %s, mean rel err %.2e %s" % (
+        rows.append(run_case(name, c, ext, repeats=args.repeats, cold=args.cold, clocks=args.clocks))
+        print("%-5s int%d K=%d S=%d M=%d B=%d g=%d %s: %.2f us, %s, mean rel err %.2e %s%s" % (
             name, bits, K, S, M, B, group, "16:32" if sparse else "dense", rows[-1]["quant_event_us"],
-            rows[-1]["rate"], rows[-1]["err_quant"], "ok" if rows[-1]["ok"] else "FAIL"), flush=True)
+            rows[-1]["rate"], rows[-1]["err_quant"], "ok" if rows[-1]["ok"] else "FAIL",
+            ", shader clock under load %s MHz (vendor fp16 GEMM: %s)" % (rows[-1]["sclk_mhz"], rows[-1]["fp16_sclk_mhz"])
+            if args.clocks > 0 else ""), flush=True)
         del c
         torch.cuda.empty_cache()
     print()
