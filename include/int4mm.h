@@ -31,6 +31,16 @@
  *                             scale <  0: w = fp16_fma(+-2^(q & (2^(bits-1)-1)), -s, z),
  *                             sign = top bit of the code.
  *   multiplier, outs        : fp16 [B, M, K] and [B, M, S], contiguous.
+ *
+ * Numerics of the products.  "Bit-exact" above is about the formats and the helpers
+ * (pack, unpack, dequantize).  int4mm_matmul with 17 or more rows of states multiplies
+ * exactly those fp16 weights and accumulates in fp32.  int4mm_matvec and the few-row
+ * kernels behind both products (2..16 rows, and up to 96 on some shapes) do not round
+ * per weight: they accumulate sum(x * q) and sum(x) in fp32 and apply scale and zero
+ * once per group, y += s * (sum(x * q) - z * sum(x)), which is the exact value of
+ * sum(x * (q - z) * s) up to fp32 rounding -- closer to the true product than the
+ * reference's fp16(fp16(q - z) * s) weights, but not the same bits.  Results are a
+ * deterministic function of the inputs and the shape (no atomics on data).
  */
 #ifndef INT4MM_H
 #define INT4MM_H
@@ -88,6 +98,11 @@ INT4MM_API int int4mm_tune(int key, int64_t value);
  *   dense : R * 32 == K * bits         sparse (bits == 4) : R * 16 == K
  *   K % 64 == 0, S % 64 == 0 (README.md:9), B, M >= 1 (B*M*S == 0 returns OK)
  *   group_size < 0 (one group) or group_size % 64 == 0; g * G >= K
+ * Two limits the reference does not have:
+ *   int4mm_matvec: K <= 458752 (INT4MM_ERR_SHAPE beyond: a workgroup stages the states
+ *   of its K range in 64 KB of LDS, 224 units of 64 rows, and K is cut at most 32 ways);
+ *   int4mm_matvec needs a workspace of int4mm_workspace_bytes(S) bytes even for shapes it
+ *   would not split (INT4MM_ERR_WORKSPACE without one; it does not fall back).
  */
 typedef struct int4mm_shape {
     int64_t batch;        /* B */
