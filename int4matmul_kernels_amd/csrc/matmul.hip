@@ -288,7 +288,8 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 2) void matmul_kernel(M
 //    the barrier that closes a step orders buffer reuse only and the MFMA
 //    stream never drains while waves wait for each other.
 // The steady-state loop body has no branches; a tile that contains exponent-mode
-// groups takes a plain loop with the general decode instead.
+// groups takes a second pipelined loop whose decode serves either mode (dense formats, 256-column
+// tiles) or a plain loop with the general decode (the others).
 constexpr int PK = 32;            // K per step of the pipelined kernel
 
 // One 16-byte chunk = 8 consecutive k of one column.  `bits` holds its 8 codes,
@@ -327,6 +328,58 @@ __device__ __forceinline__ h16x8 dequant_chunk_fast(uint32_t bits, h16x2 negz, h
         }
         return bitcast<h16x8>(r);
     }
+}
+
+// Either mode, chosen per thread (a thread decodes one column, and the mode belongs to a
+// (group, column)), without a branch: bit-exact with dequant_code in both.  Shared tail
+//     A = P + N (one rounding),  w = fma(A, B, C) (one rounding)
+// linear:   P = q, N = -z, B = s, C = -0:  fp16(q - z), then fp16(. * s) -- adding -0 changes nothing
+// exponent: P = +-2^e, N = -0, B = -s, C = z:  the reference's single-rounded fma (matmul.cuh:127-136)
+// +-2^e comes from the pair's magic-number word {2^a | q_even, 2^b | q_odd << BITS}: a packed
+// 16-bit multiply moves both codes to bits 10.. of their halves (the magic bits leave through the
+// top), the low BITS - 1 bits are the exponent field's increment over 15, the top bit is the sign.
+typedef uint16_t u16x2 __attribute__((ext_vector_type(2)));
+template <int BITS>
+__device__ __forceinline__ h16x2 expo_pair(uint32_t h) {
+    const u16x2 mul = {(uint16_t)1024, (uint16_t)(1u << (10 - BITS))};
+    const uint32_t m = bitcast<uint32_t>(bitcast<u16x2>(h) * mul);
+    constexpr uint32_t E1 = ((1u << (BITS - 1)) - 1u) << 10, EMASK = E1 | (E1 << 16);
+    const uint32_t magnitude = (m & EMASK) + 0x3C003C00u;
+    return as_h2(((m << (6 - BITS)) & 0x80008000u) | magnitude);
+}
+
+template <int BITS>
+__device__ __forceinline__ h16x8 dequant_chunk_mixed(uint32_t bits, bool expo, h16x2 negz, h16x2 s2) {
+    const h16x2 minus0 = as_h2(0x80008000u);
+    const h16x2 N = expo ? minus0 : negz, B = expo ? -s2 : s2, C = expo ? -negz : minus0;
+    uint32_t h[4];
+    h16x2 unmagic;
+    if constexpr (BITS == 4) {
+        const uint32_t MSK = vgpr_const(0x00F0000Fu), MAGIC = vgpr_const(0x54006400u);
+        unmagic = h16x2{(h16)-1024.0f, (h16)-64.0f};
+        const uint32_t lo = __builtin_amdgcn_perm(bits, bits, 0x01000100u);
+        const uint32_t hi = __builtin_amdgcn_perm(bits, bits, 0x03020302u);
+        h[0] = (lo & MSK) | MAGIC; h[1] = ((lo >> 8) & MSK) | MAGIC;
+        h[2] = (hi & MSK) | MAGIC; h[3] = ((hi >> 8) & MSK) | MAGIC;
+    } else {
+        constexpr uint32_t MSK = BITS == 2 ? 0x000C0003u : 0x00380007u;
+        constexpr uint32_t MAGIC = BITS == 2 ? 0x5C006400u : 0x58006400u;
+        unmagic = h16x2{(h16)-1024.0f, BITS == 2 ? (h16)-256.0f : (h16)-128.0f};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t u = bits >> (2 * BITS * j);
+            h[j] = (__builtin_amdgcn_perm(u, u, 0x01000100u) & MSK) | MAGIC;
+        }
+    }
+    u32x4 r;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const h16x2 q = as_h2(h[j]) + unmagic;             // exact: {q_even, q_odd}
+        const h16x2 P = expo ? expo_pair<BITS>(h[j]) : q;
+        const h16x2 A = P + N;
+        r[j] = as_u32(__builtin_elementwise_fma(A, B, C));
+    }
+    return bitcast<h16x8>(r);
 }
 
 // 16:32 sparse int4.  `v` holds the (up to 8) kept codes of one 8-row chunk as
@@ -574,7 +627,7 @@ __device__ __forceinline__ void pipe_tile(const MatmulArgs& a, const int m0, con
     // Does any (group, column) of this tile use exponent quantisation (scale < 0
     // or NaN)?  One pass over the tile's scales (a few KB); the answer is
     // workgroup-uniform and selects between the pipelined loop, whose decode is
-    // the branch-free linear one, and a plain loop with the general decode.
+    // the branch-free linear one, and the loops that also serve exponent groups.
     int& any_expo = *reinterpret_cast<int*>(Bs);          // borrowed before the pipeline starts
     __syncthreads();
     if constexpr (SPARSE) {
@@ -761,6 +814,94 @@ __device__ __forceinline__ void pipe_tile(const MatmulArgs& a, const int m0, con
                 run(std::integral_constant<int, 0>{});
             } else {
                 run(std::integral_constant<int, 1>{});
+            }
+        }
+    } else if constexpr (!SPARSE && NW == 4) {
+        // A tile with exponent-mode groups: the same three-stage pipeline (in the plain order of a
+        // step: fragments, loads, decode between the MFMAs, stores, barrier) with the decode that
+        // serves either mode per thread.  (256-column tiles only: in the 128-column kernel, which
+        // keeps two workgroups per compute unit, this loop does not fit the registers, and its
+        // spills slowed the linear loop down as well.)
+        Cursor cur = cursor_at(kt0);
+        const int gu2 = a.group_units * 2;
+        auto advance = [&]() {
+            const int more = min(last - cur.kt, 1);
+            const int wrap = cur.left == 1 ? more : 0;
+            cur.kt += more;
+            cur.w += more * b_step;
+            cur.sz += wrap * g_step;
+            cur.left += wrap * gu2 - more;
+        };
+        uint32_t a_cur = (uint32_t)kt0 * (PK * 2);
+        int a_kt = kt0;
+        auto advance_a = [&]() {
+            const int more = min(last - a_kt, 1);
+            a_kt += more;
+            a_cur += more * (PK * 2);
+        };
+        auto write_b_mixed = [&](const Stage& s, int stage, int q) {
+            const h16x2 s2 = stage_scale(s);
+            const bool expo = !(s2.x >= (h16)0.0f);
+            const h16x8 w = dequant_chunk_mixed<BITS>(chunk_bits(s, q), expo, stage_negzero(s), s2);
+            *reinterpret_cast<h16x8*>(&Bs[stage * B_STAGE + ((bhb * 2 + q) * BN + bn) * 8]) = w;
+        };
+        Stage r[3];
+        AStage ra[2];
+        h16x8 fa[2][TM], fb[2][TN];
+        auto body_mixed = [&](int b, AStage& ra_new, const AStage& ra_wr, Stage& r_new, const Stage& r_dec) {
+            const int b1 = (b + 1) % P_STAGES, b2 = (b + 2) % P_STAGES;
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks) {
+                if (ks == 0) load_frags(b, 1, fa[1], fb[1]);
+                else load_frags(b1, 0, fa[0], fb[0]);
+                if (ks == 0) {
+                    load_a(ra_new, a_cur);             // step kt + 3
+                    load_b(r_new, cur);                // step kt + 4
+                    advance_a();
+                    advance();
+                    write_b_mixed(r_dec, b2, 0);
+                    write_b_mixed(r_dec, b2, 1);
+                } else {
+                    write_a(ra_wr, b2);
+                }
+                mfma_slice(fa[ks], fb[ks]);
+                if (ks == 0) {
+                    __builtin_amdgcn_sched_group_barrier(0x100, TM + TN, 0);
+#pragma unroll
+                    for (int e = 0; e < TM * TN; ++e) {
+                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                        __builtin_amdgcn_sched_group_barrier(0x002, TM == 4 ? 14 : 28, 0);
+                        if (e < A_LOADS + NWORDS + 2) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+                    }
+                    __builtin_amdgcn_sched_group_barrier(0x200, 2, 0);
+                } else {
+                    __builtin_amdgcn_sched_group_barrier(0x100, TM + TN, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x200, A_LOADS, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x008, TM * TN - 1, 0);
+                }
+            }
+            __builtin_amdgcn_s_waitcnt(0xC07F);      // lgkmcnt(0) only
+            __builtin_amdgcn_s_barrier();
+        };
+        load_a(ra[0], a_cur); advance_a();
+        load_a(ra[1], a_cur); advance_a();
+        load_b(r[0], cur); advance();
+        load_b(r[1], cur); advance();
+        write_a(ra[0], 0);
+        write_a(ra[1], 1);
+        load_a(ra[0], a_cur); advance_a();              // step 2
+#pragma unroll
+        for (int q = 0; q < 2; ++q) { write_b_mixed(r[0], 0, q); write_b_mixed(r[1], 1, q); }
+        load_b(r[2], cur); advance();                   // step 2
+        load_b(r[0], cur); advance();                   // step 3
+        __syncthreads();
+        load_frags(0, 0, fa[0], fb[0]);
+        for (int kt = 0; kt < ktiles; kt += 6) {
+#pragma unroll
+            for (int u = 0; u < 6; ++u) {
+                if (u > 0 && kt + u >= ktiles) break;
+                body_mixed(u % 3, ra[(u + 1) % 2], ra[u % 2], r[(u + 1) % 3], r[(u + 2) % 3]);
             }
         }
     } else {

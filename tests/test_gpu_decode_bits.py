@@ -28,14 +28,15 @@ def H():
     return helpers
 
 
-def _problem(bits, sparse, K, S, g, seed):
+def _problem(bits, sparse, K, S, g, seed, expo=True):
     kw = {}
     if bits != 4:
         kw = dict(scale_range=(0.004, 0.08), zero_const=3.5 if bits == 3 else 1.5)
     p = O.make_problem(K=K, S=S, M=K, bits=bits, group_size=g, sparse=sparse, seed=seed, **kw)
     sc = p["scales"]
-    sc[1, 3::7] *= np.float16(-1)                # exponent quantisation in some columns of one group
-    sc[:, 64:72] *= np.float16(-1)               # and in a few columns throughout
+    if expo:
+        sc[1, 3::7] *= np.float16(-1)            # exponent quantisation in some columns of one group
+        sc[:, 64:72] *= np.float16(-1)           # and in a few columns throughout
     if bits == 4 and not sparse:
         p["zeros"][0, :16] = np.float16(7.0)     # integer zero: some weights are exactly 0
     p["states"] = np.eye(K, dtype=np.float16)[None]
@@ -53,11 +54,15 @@ def _assert_same_bits(got, want, what):
 
 @pytest.mark.parametrize("bits,sparse", FORMATS)
 @pytest.mark.parametrize("variant", [1, 3, 5, 6, 7, 9])
-def test_tile_kernels_return_the_dequantised_weights(H, bits, sparse, variant):
+@pytest.mark.parametrize("expo", [False, True], ids=["linear", "mixed"])
+def test_tile_kernels_return_the_dequantised_weights(H, bits, sparse, variant, expo):
+    """`linear`: no exponent group anywhere, so the pipelined kernels run their linear-only loop;
+    `mixed`: every tile holds groups of both modes and takes the loop (or, for the 128-column and
+    16:32 tiles, the plain loop) that decodes either."""
     if variant == 5 and sparse:
         pytest.skip("256 x 128 tiles serve the dense formats only")
     K, S, g = 512, 512, 128
-    p = _problem(bits, sparse, K, S, g, seed=70 + bits)
+    p = _problem(bits, sparse, K, S, g, seed=70 + bits, expo=expo)
     want = O.dequantize_matrix(bits, p["matrix"], p["scales"], p["zeros"], g, p["sparse_mask"])
     d = H.dev_problem(p)
     H.capi.tune(3, variant)

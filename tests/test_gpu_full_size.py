@@ -118,3 +118,23 @@ def test_sparse_matvec_full_size(H):
         w32 = np.where(keep[:, cols], (q.astype(np.float32) - z.astype(np.float32)) * s.astype(np.float32), np.float32(0))
         f32[:, cols] = O.matmul_fp32(x.reshape(1, K), w32)
     H.assert_product_close(got, exact.reshape(1, 1, S), f32.reshape(1, 1, S))
+
+
+@pytest.mark.parametrize("bits", [4, 3])
+def test_mixed_quantisation_modes_matmul_full_size(H, bits):
+    """M = 2048, K = 5120, S = 20480 with exponent-mode groups scattered over the matrix (negative scale:
+    matmul.cuh:414-428): one whole group row, every third column of another, single entries elsewhere.
+    Every 256 x 256 tile then contains both modes and takes the pipelined loop whose decode serves either."""
+    K, S, g, M = 5120, 20480, 128, 2048
+    p = O.make_problem(K=K, S=S, M=M, bits=bits, group_size=g, seed=3, zero_range=(0.0, 4.0))
+    sc = p["scales"].copy()
+    sc[7] = -sc[7]
+    sc[19, ::3] = -sc[19, ::3]
+    sc[np.arange(40), np.arange(40) * 509 % S] *= np.float16(-1)
+    p = dict(p, scales=sc)
+    out = H.run_capi(p, H.dev_problem(p), "mtx")
+    rows = np.linspace(0, M - 1, 24).astype(int)
+    # (the fp32 dequantise-then-matmul oracle is linear-mode only: the exact product on the fp16 weights is the check)
+    w16 = O.dequantize_matrix(bits, p["matrix"], p["scales"], p["zeros"], g, None)
+    assert O.max_rel_error(O.matmul_exact(p["states"][0, rows], w16), out[0, rows], floor_frac=H.FLOOR_EXACT_MTX) < H.TOL_EXACT_MTX
+    assert np.all(np.isfinite(out.astype(np.float32)))
