@@ -76,6 +76,12 @@ template <int BITS, bool SPARSE>
 __device__ __forceinline__ void load_unit(Unit<BITS, SPARSE>& u, const MatvecArgs& a, int unit, int col) {
     constexpr int ROWS = Fmt<BITS, SPARSE>::ROWS, MROWS = Fmt<BITS, SPARSE>::MROWS;
     const int64_t S = a.S;
+    // scale / zero first: loads return in order, so the unit is complete when its last weight
+    // row arrives instead of two small requests to other pages later
+    const int64_t gofs = (int64_t)(unit / a.group_units) * S + col;
+    u.sc = *reinterpret_cast<const u32x2*>(a.scales + gofs);
+    u.ze = *reinterpret_cast<const u32x2*>(a.zeros + gofs);
+    __builtin_amdgcn_sched_barrier(0);
     const uint32_t* p = a.matrix + (int64_t)unit * ROWS * S + col;
 #pragma unroll
     for (int r = 0; r < ROWS; ++r) u.w[r] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p + r * S));
@@ -84,9 +90,6 @@ __device__ __forceinline__ void load_unit(Unit<BITS, SPARSE>& u, const MatvecArg
 #pragma unroll
         for (int r = 0; r < MROWS; ++r) u.m[r] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(q + r * S));
     }
-    const int64_t gofs = (int64_t)(unit / a.group_units) * S + col;
-    u.sc = *reinterpret_cast<const u32x2*>(a.scales + gofs);
-    u.ze = *reinterpret_cast<const u32x2*>(a.zeros + gofs);
 }
 
 // (w & mask) | magic is one VALU op (v_and_or_b32) only when both constants sit
