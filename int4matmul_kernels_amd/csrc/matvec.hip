@@ -106,6 +106,30 @@ __device__ __forceinline__ uint32_t and_or(uint32_t w, uint32_t mask, uint32_t m
     return (w & mask) | magic;
 }
 
+// Exponent quantisation on the same operands.  A magic-number pair holds its two codes inside
+// the mantissas, at offsets o with 2^(10 - o) the pair's magic offsets; a packed 16-bit multiply
+// by those offsets moves both codes to bits 10.. of their halves (whatever the magic bits turn
+// into lies above and is masked away).  The code's low BITS - 1 bits are then the exponent
+// field's increment over 15 (2^0) and its top bit is the sign: the half is +-2^(code's low bits),
+// the value the exponent mode multiplies by (matmul.cuh:127-136).
+typedef uint16_t u16x2 __attribute__((ext_vector_type(2)));
+template <int BITS>
+__device__ __forceinline__ uint32_t expo_operand(uint32_t h, uint32_t offsets) {
+    const uint32_t m = bitcast<uint32_t>(bitcast<u16x2>(h) * bitcast<u16x2>(offsets));
+    constexpr uint32_t E1 = ((1u << (BITS - 1)) - 1u) << 10, EMASK = E1 | (E1 << 16);
+    const uint32_t magnitude = (m & EMASK) + 0x3C003C00u;
+    return ((m << (6 - BITS)) & 0x80008000u) | magnitude;
+}
+// operand of the matrix core for one pair: {2^a + q, 2^b + q'} (linear mode, offsets removed
+// later) or {+-2^e, +-2^e'} (exponent mode, nothing to remove); `offsets` = {2^a, 2^b} as integers
+template <int BITS, bool EXPO>
+__device__ __forceinline__ uint32_t operand(uint32_t w, uint32_t mask, uint32_t magic, uint32_t offsets) {
+    const uint32_t h = and_or(w, mask, magic);
+    if constexpr (EXPO) return expo_operand<BITS>(h, offsets);
+    else return h;
+}
+__host__ __device__ constexpr uint32_t off2(uint32_t lo, uint32_t hi) { return lo | (hi << 16); }
+
 // ---- fast paths.  xp points at the unit's staged states (LDS).
 //
 // The multiply-accumulate itself runs on the matrix core, which is otherwise
@@ -133,9 +157,11 @@ __device__ __forceinline__ f32x4 mma4(uint32_t a0, uint32_t a1, uint32_t b0, uin
 #ifndef MV_NCOL
 #define MV_NCOL 2
 #endif
+template <bool EXPO = false>
 __device__ __forceinline__ void unit_fast(const Unit<4, false>& u, const h16* xp, f32x4 acc[4]) {
     const uint32_t M0 = in_vgpr(0x000F000Fu), M1 = in_vgpr(0x00F000F0u);
     const uint32_t G0 = in_vgpr(0x64006400u), G1 = in_vgpr(0x54005400u);
+    constexpr uint32_t O0 = off2(1024, 1024), O1 = off2(64, 64);
 #pragma unroll
     for (int c0 = 0; c0 < 4; c0 += MV_NCOL) {
 #pragma unroll
@@ -144,8 +170,8 @@ __device__ __forceinline__ void unit_fast(const Unit<4, false>& u, const h16* xp
 #pragma unroll
             for (int c = c0; c < c0 + MV_NCOL; ++c) {
                 const uint32_t w = u.w[r][c], w8 = w >> 8;
-                acc[c] = mma4(p.x, p.y, and_or(w, M0, G0), and_or(w, M1, G1), acc[c]);
-                acc[c] = mma4(p.z, p.w, and_or(w8, M0, G0), and_or(w8, M1, G1), acc[c]);
+                acc[c] = mma4(p.x, p.y, operand<4, EXPO>(w, M0, G0, O0), operand<4, EXPO>(w, M1, G1, O1), acc[c]);
+                acc[c] = mma4(p.z, p.w, operand<4, EXPO>(w8, M0, G0, O0), operand<4, EXPO>(w8, M1, G1, O1), acc[c]);
             }
         }
     }
@@ -155,7 +181,9 @@ __device__ __forceinline__ void unit_fast(const Unit<4, false>& u, const h16* xp
 // offsets 0,2,4,6,8 fit the mantissa (magic 2^(10-o)); codes 5,6,7 / 13,14,15
 // come down to offsets 0,2,4 after a shift by 10.  Staged states per packed row:
 // {x_j, x_{j+8}} for j = 0..7.  off_k by k mod 8: 1024,256,64,16,4,1024,256,64.
+template <bool EXPO = false>
 __device__ __forceinline__ void unit_fast(const Unit<2, false>& u, const h16* xp, f32x4 acc[4]) {
+    constexpr uint32_t O0 = off2(1024, 1024), O1 = off2(256, 256), O2 = off2(64, 64), O3 = off2(16, 16), O4 = off2(4, 4);
     const uint32_t M0 = in_vgpr(0x00030003u), M1 = in_vgpr(0x000C000Cu), M2 = in_vgpr(0x00300030u),
                    M3 = in_vgpr(0x00C000C0u), M4 = in_vgpr(0x03000300u);
     const uint32_t G0 = in_vgpr(0x64006400u), G1 = in_vgpr(0x5C005C00u), G2 = in_vgpr(0x54005400u),
@@ -167,10 +195,10 @@ __device__ __forceinline__ void unit_fast(const Unit<2, false>& u, const h16* xp
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
             const uint32_t w = u.w[r][c], w10 = w >> 10;
-            acc[c] = mma4(pa.x, pa.y, and_or(w, M0, G0), and_or(w, M1, G1), acc[c]);
-            acc[c] = mma4(pa.z, pa.w, and_or(w, M2, G2), and_or(w, M3, G3), acc[c]);
-            acc[c] = mma4(pb.x, pb.y, and_or(w, M4, G4), and_or(w10, M0, G0), acc[c]);
-            acc[c] = mma4(pb.z, pb.w, and_or(w10, M1, G1), and_or(w10, M2, G2), acc[c]);
+            acc[c] = mma4(pa.x, pa.y, operand<2, EXPO>(w, M0, G0, O0), operand<2, EXPO>(w, M1, G1, O1), acc[c]);
+            acc[c] = mma4(pa.z, pa.w, operand<2, EXPO>(w, M2, G2, O2), operand<2, EXPO>(w, M3, G3, O3), acc[c]);
+            acc[c] = mma4(pb.x, pb.y, operand<2, EXPO>(w, M4, G4, O4), operand<2, EXPO>(w10, M0, G0, O0), acc[c]);
+            acc[c] = mma4(pb.z, pb.w, operand<2, EXPO>(w10, M1, G1, O1), operand<2, EXPO>(w10, M2, G2, O2), acc[c]);
         }
     }
 }
@@ -191,7 +219,9 @@ __device__ constexpr int I3_HI[18] = {5, 6, 7, 13, 14, 15, 21, 22, 23, 29, 30, 3
 __device__ constexpr float I3_OFF[32] = {512, 64, 8, 1024, 1024, 1024, 128, 16, 512, 64, 8, 32, 1024, 1024, 128, 16,
                                          512, 64, 8, 32, 1024, 1024, 128, 16, 512, 64, 8, 32, 1024, 1024, 128, 16};
 
+template <bool EXPO = false>
 __device__ __forceinline__ void unit_fast(const Unit<3, false>& u, const h16* xp, f32x4 acc[4]) {
+    constexpr uint32_t OA1 = off2(512, 1024), OA2 = off2(64, 128), OA3 = off2(8, 16), OL = off2(1024, 32), OS = off2(1024, 1024);
     const uint32_t MA1 = in_vgpr(0x0007000Eu), GA1 = in_vgpr(0x64006000u);   // {512 + c, 1024 + c5}
     const uint32_t MA2 = in_vgpr(0x00380070u), GA2 = in_vgpr(0x58005400u);   // {64 + c1, 128 + c6}
     const uint32_t MA3 = in_vgpr(0x01C00380u), GA3 = in_vgpr(0x4C004800u);   // {8 + c2, 16 + c7}
@@ -212,15 +242,15 @@ __device__ __forceinline__ void unit_fast(const Unit<3, false>& u, const h16* xp
                            l2 = __builtin_amdgcn_alignbit(w2, w1, 28);
             const uint32_t s3 = w0 >> 9, s28 = w2 >> 20;
             f32x4 r = acc[c];
-            r = mma4(p0.x, p0.y, and_or(a0, MA1, GA1), and_or(a0, MA2, GA2), r);
-            r = mma4(p0.z, p0.w, and_or(a0, MA3, GA3), and_or(a1, MA1, GA1), r);
-            r = mma4(p1.x, p1.y, and_or(a1, MA2, GA2), and_or(a1, MA3, GA3), r);
-            r = mma4(p1.z, p1.w, and_or(a2, MA1, GA1), and_or(a2, MA2, GA2), r);
-            r = mma4(p2.x, p2.y, and_or(a2, MA3, GA3), and_or(a3, MA1, GA1), r);
-            r = mma4(p2.z, p2.w, and_or(a3, MA2, GA2), and_or(a3, MA3, GA3), r);
-            r = mma4(p3.x, p3.y, and_or(l0, ML, GL), and_or(l1, ML, GL), r);
-            r = mma4(p3.z, p3.w, and_or(l2, ML, GL), and_or(s3, MS, GS), r);
-            const uint32_t last = and_or(s28, MS, GS);
+            r = mma4(p0.x, p0.y, operand<3, EXPO>(a0, MA1, GA1, OA1), operand<3, EXPO>(a0, MA2, GA2, OA2), r);
+            r = mma4(p0.z, p0.w, operand<3, EXPO>(a0, MA3, GA3, OA3), operand<3, EXPO>(a1, MA1, GA1, OA1), r);
+            r = mma4(p1.x, p1.y, operand<3, EXPO>(a1, MA2, GA2, OA2), operand<3, EXPO>(a1, MA3, GA3, OA3), r);
+            r = mma4(p1.z, p1.w, operand<3, EXPO>(a2, MA1, GA1, OA1), operand<3, EXPO>(a2, MA2, GA2, OA2), r);
+            r = mma4(p2.x, p2.y, operand<3, EXPO>(a2, MA3, GA3, OA3), operand<3, EXPO>(a3, MA1, GA1, OA1), r);
+            r = mma4(p2.z, p2.w, operand<3, EXPO>(a3, MA2, GA2, OA2), operand<3, EXPO>(a3, MA3, GA3, OA3), r);
+            r = mma4(p3.x, p3.y, operand<3, EXPO>(l0, ML, GL, OL), operand<3, EXPO>(l1, ML, GL, OL), r);
+            r = mma4(p3.z, p3.w, operand<3, EXPO>(l2, ML, GL, OL), operand<3, EXPO>(s3, MS, GS, OS), r);
+            const uint32_t last = operand<3, EXPO>(s28, MS, GS, OS);
             r = mma4(p4.x, p4.y, last, last, r);          // second pair is unused: its states are zero
             acc[c] = r;
         }
@@ -635,17 +665,36 @@ void matvec_kernel(MatvecArgs a) {
     }
 
     if constexpr (FAST) {
-        // exponent-mode columns: second pass with the general decoder, only where needed
+        // exponent-mode columns: a second pass over the units that have any (the group's scales
+        // are looked at first; most units are skipped).  Dense formats run the same operands
+        // through the exponent decode -- no offsets to remove, y += z * sum(x) - s * sum(x * +-2^e);
+        // 16:32 takes the general decoder.
         if (__builtin_amdgcn_ballot_w64(need_general) != 0 && work) {
             for (int v = wg_u0 + grp; v < wg_u1; v += ng) {
+                const u32x2 sc2 = *reinterpret_cast<const u32x2*>(a.scales + (int64_t)(v / a.group_units) * a.S + col);
+                const h16x2 s01 = as_h2(sc2.x), s23 = as_h2(sc2.y);
+                const bool any = !(s01.x >= (h16)0.f) | !(s01.y >= (h16)0.f) | !(s23.x >= (h16)0.f) | !(s23.y >= (h16)0.f);
+                if (__builtin_amdgcn_ballot_w64(any) == 0) continue;
                 load_unit(ua, a, v, col);
-                float sc[4], ze[4], acc[4], xsv[4];
+                float sc[4], ze[4];
                 bool expo[4];
                 unpack_params(ua.sc, ua.ze, sc, ze, expo);
-                if (!(expo[0] | expo[1] | expo[2] | expo[3])) continue;
-                unit_generic<BITS, SPARSE>(ua, a.x + v * 64, expo, acc, xsv);
+                if constexpr (!SPARSE) {
+                    f32x4 acc[4];
 #pragma unroll
-                for (int c = 0; c < 4; ++c) y[c] += expo[c] ? ze[c] * xsv[c] - sc[c] * acc[c] : 0.f;
+                    for (int c = 0; c < 4; ++c) acc[c] = f32x4{0.f, 0.f, 0.f, 0.f};
+                    const int lu = v - wg_u0;
+                    unit_fast<true>(ua, xs + lu * (Fmt<BITS, SPARSE>::XS / 2), acc);
+                    const float xsum = sums[lu * 2];
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) y[c] += expo[c] ? ze[c] * xsum - sc[c] * acc[c][0] : 0.f;
+                } else {
+                    if (!(expo[0] | expo[1] | expo[2] | expo[3])) continue;
+                    float acc[4], xsv[4];
+                    unit_generic<BITS, SPARSE>(ua, a.x + v * 64, expo, acc, xsv);
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) y[c] += expo[c] ? ze[c] * xsv[c] - sc[c] * acc[c] : 0.f;
+                }
             }
         }
     }

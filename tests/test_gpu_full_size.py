@@ -138,3 +138,27 @@ def test_mixed_quantisation_modes_matmul_full_size(H, bits):
     w16 = O.dequantize_matrix(bits, p["matrix"], p["scales"], p["zeros"], g, None)
     assert O.max_rel_error(O.matmul_exact(p["states"][0, rows], w16), out[0, rows], floor_frac=H.FLOOR_EXACT_MTX) < H.TOL_EXACT_MTX
     assert np.all(np.isfinite(out.astype(np.float32)))
+
+
+@pytest.mark.parametrize("bits", [4, 3, 2])
+def test_mixed_quantisation_modes_matvec_full_size(H, bits):
+    """K = 5120, S = 20480, M = 1 with exponent-mode groups: one whole group row, every third column of another,
+    single entries elsewhere.  The matvec's first pass skips those (group, column) pairs; its second pass visits
+    only the units that hold any and decodes them with the exponent form of the same operands."""
+    K, S, g = 5120, 20480, 128
+    kw = {} if bits == 4 else dict(scale_range=(0.004, 0.08), zero_const=3.5 if bits == 3 else 1.5)
+    p = O.make_problem(K=K, S=S, M=1, bits=bits, group_size=g, seed=4, **kw)
+    sc = p["scales"].copy()
+    sc[7] = -sc[7]
+    sc[19, ::3] = -sc[19, ::3]
+    sc[np.arange(40), np.arange(40) * 509 % S] *= np.float16(-1)
+    p = dict(p, scales=sc)
+    got = H.run_capi(p, H.dev_problem(p), "vec")
+    x = p["states"].reshape(1, K)
+    exact = np.empty((1, S), np.float64)
+    for c0 in range(0, S, 2048):
+        cols = slice(c0, c0 + 2048)
+        w16 = O.dequantize_matrix(bits, p["matrix"][:, cols], sc[:, cols], p["zeros"][:, cols], g, None)
+        exact[:, cols] = O.matmul_exact(x, w16)
+    exact = exact.reshape(1, 1, S)
+    H.assert_product_close(got, exact, exact.astype(np.float32))
