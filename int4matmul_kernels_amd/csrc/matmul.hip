@@ -624,6 +624,40 @@ __device__ __forceinline__ void pipe_tile(const MatmulArgs& a, const int m0, con
     const int ktiles = SPLIT ? min(ksteps, kt0 + per_split) - kt0 : ksteps;
     const int last = kt0 + ktiles - 1;
 
+    // Cursors of the loads: weights run four K steps ahead of the MFMAs, states
+    // three; both stop at the last step (the surplus loads re-read it, unused).
+    Cursor cur = cursor_at(kt0);
+    // (selects instead of branches: a branch here would split the scheduling
+    // region of the step and invite the compiler to reuse the previous step's
+    // scale / zero registers, which makes the step wait for its newest loads)
+    // (plain integer arithmetic on purpose: conditions kept as booleans come out as
+    // 64-bit lane-mask operations, several scalar instructions each)
+    const int gu2 = a.group_units * 2;
+    auto advance = [&]() {
+        const int more = min(last - cur.kt, 1);                  // 1 until the last step is reached
+        const int wrap = cur.left == 1 ? more : 0;
+        cur.kt += more;
+        cur.w += more * b_step;
+        if constexpr (SPARSE) cur.m += more * m_step;
+        cur.sz += wrap * g_step;
+        cur.left += wrap * gu2 - more;
+    };
+    uint32_t a_cur = (uint32_t)kt0 * (PK * 2);
+    int a_kt = kt0;
+    auto advance_a = [&]() {
+        const int more = min(last - a_kt, 1);
+        a_kt += more;
+        a_cur += more * (PK * 2);
+    };
+    Stage r[3];
+    AStage ra[2];
+    // the first two steps' operands are requested before the look at the scales below, whose
+    // round trip to memory they then share
+    load_a(ra[0], a_cur); advance_a();
+    load_a(ra[1], a_cur); advance_a();
+    load_b(r[0], cur); advance();
+    load_b(r[1], cur); advance();
+
     // Does any (group, column) of this tile use exponent quantisation (scale < 0
     // or NaN)?  One pass over the tile's scales (a few KB); the answer is
     // workgroup-uniform and selects between the pipelined loop, whose decode is
@@ -641,9 +675,27 @@ __device__ __forceinline__ void pipe_tile(const MatmulArgs& a, const int m0, con
     if (t == 0) any_expo = 0;
     __syncthreads();
     {
+        // the tile's scales are `groups` rows of BN / 2 aligned 32-bit words; the threads share them
+        // out and fetch four words each per trip, all in flight together (one round trip to
+        // memory instead of one per group)
         bool bad = false;
         const int groups = (ksteps + a.group_units * 2 - 1) / (a.group_units * 2);
-        for (int g = bhb; g < groups; g += 2) bad |= !(a.scales[(int64_t)g * a.S + bcol] >= (h16)0.0f);
+        const int total = groups * (BN / 2);
+        const uint32_t* tile_scales = reinterpret_cast<const uint32_t*>(a.scales + s0);
+        const int64_t row_words = a.S / 2;
+        for (int i0 = t; i0 < total; i0 += 4 * T) {
+            uint32_t v[4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const int i = min(i0 + k * T, total - 1);
+                v[k] = tile_scales[(int64_t)(i / (BN / 2)) * row_words + i % (BN / 2)];
+            }
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const h16x2 h = as_h2(v[k]);
+                bad |= !(h.x >= (h16)0.0f) | !(h.y >= (h16)0.0f);
+            }
+        }
         if (__builtin_amdgcn_ballot_w64(bad) != 0 && lane == 0) any_expo = 1;
     }
     __syncthreads();
@@ -651,33 +703,6 @@ __device__ __forceinline__ void pipe_tile(const MatmulArgs& a, const int m0, con
     __syncthreads();
 
     if (!tile_has_expo) {
-        // Cursors of the loads: weights run four K steps ahead of the MFMAs, states
-        // three; both stop at the last step (the surplus loads re-read it, unused).
-        Cursor cur = cursor_at(kt0);
-        // (selects instead of branches: a branch here would split the scheduling
-        // region of the step and invite the compiler to reuse the previous step's
-        // scale / zero registers, which makes the step wait for its newest loads)
-        // (plain integer arithmetic on purpose: conditions kept as booleans come out as
-        // 64-bit lane-mask operations, several scalar instructions each)
-        const int gu2 = a.group_units * 2;
-        auto advance = [&]() {
-            const int more = min(last - cur.kt, 1);                  // 1 until the last step is reached
-            const int wrap = cur.left == 1 ? more : 0;
-            cur.kt += more;
-            cur.w += more * b_step;
-            if constexpr (SPARSE) cur.m += more * m_step;
-            cur.sz += wrap * g_step;
-            cur.left += wrap * gu2 - more;
-        };
-        uint32_t a_cur = (uint32_t)kt0 * (PK * 2);
-        int a_kt = kt0;
-        auto advance_a = [&]() {
-            const int more = min(last - a_kt, 1);
-            a_kt += more;
-            a_cur += more * (PK * 2);
-        };
-        Stage r[3];
-        AStage ra[2];
         h16x8 fa[2][TM], fb[2][TN];         // fragments of the current and the next k slice
         // Step kt, u = kt % 6, stage b = kt % 3.  On entry: states and decoded weights
         // of steps kt, kt+1 are complete in stages b, b+1; ra[kt % 2] holds the states
@@ -776,10 +801,6 @@ __device__ __forceinline__ void pipe_tile(const MatmulArgs& a, const int m0, con
             __builtin_amdgcn_s_barrier();
             __builtin_amdgcn_sched_barrier(0);
         };
-        load_a(ra[0], a_cur); advance_a();
-        load_a(ra[1], a_cur); advance_a();
-        load_b(r[0], cur); advance();
-        load_b(r[1], cur); advance();
         write_a(ra[0], 0);
         write_a(ra[1], 1);
         load_a(ra[0], a_cur); advance_a();              // step 2
@@ -822,31 +843,12 @@ __device__ __forceinline__ void pipe_tile(const MatmulArgs& a, const int m0, con
         // serves either mode per thread.  (256-column tiles only: in the 128-column kernel, which
         // keeps two workgroups per compute unit, this loop does not fit the registers, and its
         // spills slowed the linear loop down as well.)
-        Cursor cur = cursor_at(kt0);
-        const int gu2 = a.group_units * 2;
-        auto advance = [&]() {
-            const int more = min(last - cur.kt, 1);
-            const int wrap = cur.left == 1 ? more : 0;
-            cur.kt += more;
-            cur.w += more * b_step;
-            cur.sz += wrap * g_step;
-            cur.left += wrap * gu2 - more;
-        };
-        uint32_t a_cur = (uint32_t)kt0 * (PK * 2);
-        int a_kt = kt0;
-        auto advance_a = [&]() {
-            const int more = min(last - a_kt, 1);
-            a_kt += more;
-            a_cur += more * (PK * 2);
-        };
         auto write_b_mixed = [&](const Stage& s, int stage, int q) {
             const h16x2 s2 = stage_scale(s);
             const bool expo = !(s2.x >= (h16)0.0f);
             const h16x8 w = dequant_chunk_mixed<BITS>(chunk_bits(s, q), expo, stage_negzero(s), s2);
             *reinterpret_cast<h16x8*>(&Bs[stage * B_STAGE + ((bhb * 2 + q) * BN + bn) * 8]) = w;
         };
-        Stage r[3];
-        AStage ra[2];
         h16x8 fa[2][TM], fb[2][TN];
         auto body_mixed = [&](int b, AStage& ra_new, const AStage& ra_wr, Stage& r_new, const Stage& r_dec) {
             const int b1 = (b + 1) % P_STAGES, b2 = (b + 2) % P_STAGES;
@@ -884,10 +886,6 @@ __device__ __forceinline__ void pipe_tile(const MatmulArgs& a, const int m0, con
             __builtin_amdgcn_s_waitcnt(0xC07F);      // lgkmcnt(0) only
             __builtin_amdgcn_s_barrier();
         };
-        load_a(ra[0], a_cur); advance_a();
-        load_a(ra[1], a_cur); advance_a();
-        load_b(r[0], cur); advance();
-        load_b(r[1], cur); advance();
         write_a(ra[0], 0);
         write_a(ra[1], 1);
         load_a(ra[0], a_cur); advance_a();              // step 2
