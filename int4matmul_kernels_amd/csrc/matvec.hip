@@ -840,6 +840,18 @@ static int matvec_impl(int bits, void* outs, const void* matrix, const void* mul
         if (upwg < 4) upwg = 4;
     }
     if (upwg > units_total) upwg = units_total;
+    // 160 strips x 4 splits = 640 workgroups of 4 waves leave the 256 compute units with 2 or 3
+    // workgroups each; twice the splits with half the waves are exactly 5 per compute unit, and
+    // the dense int4 kernel gains 1 - 7 % from that (measured for K = 4096 ... 11008 at S = 20480;
+    // int3 / int2 and the strips of 64 columns lose 2 - 4 %, so they keep the wider workgroups)
+    if (tuning(TUNE_MV_WAVES) <= 0 && tuning(TUNE_MV_UNITS) <= 0 && bits == 4 && sparse_mask == nullptr && lk == 2) {
+        const int s1 = (units_total + upwg - 1) / upwg, half = (upwg + 1) / 2;
+        const int s2 = (units_total + half - 1) / half;
+        if (half >= 8 && (strips * s1) % 256 != 0 && (strips * s2) % 256 == 0 && s2 <= MV_MAX_SPLITS) {
+            upwg = half;
+            waves = 2;
+        }
+    }
     int splits = (units_total + upwg - 1) / upwg;
     if (splits > MV_MAX_SPLITS) {                           // bounded slot count: more units each
         upwg = (units_total + MV_MAX_SPLITS - 1) / MV_MAX_SPLITS;

@@ -83,6 +83,28 @@ def run(K=5120, S=20480, g=128, reps=4, nsets=7, dev="cuda"):
                 print(f"workgroup end times (us): median {np.nanmedian(end[wg_live]):.2f}, "
                       f"90th percentile {np.nanpercentile(end[wg_live], 90):.2f}, max {np.nanmax(end[wg_live]):.2f}"
                       + ("" if len(first_gap) == 0 else " (non-contiguous workgroup numbering)"))
+                # by accelerator die (XCC id of the workgroup's first wave) and by K split (workgroups are
+                # numbered split-major: index = split * strips + strip)
+                wg_xcc = ((a[:, 0, 15] >> 32) & 0xF)[wg_live]
+                e = end[wg_live]
+                print("  by die:   " + "  ".join(f"{x}: {np.median(e[wg_xcc == x]):.2f} / {e[wg_xcc == x].max():.2f}"
+                                                 for x in np.unique(wg_xcc)) + "   (median / max)")
+                for k, name in ((0, "entry"), (1, "first requests issued"), (3, "unit 0 consumed")):
+                    v = rel[:, 0, k][wg_live]
+                    print(f"            {name}, median by die: " + "  ".join(
+                        f"{x}: {np.nanmedian(v[wg_xcc == x]):.2f}" for x in np.unique(wg_xcc)))
+                hw0 = a[:, 0, 15][wg_live]
+                wg_cu = ((hw0 >> 32) & 0xF) * 4096 + ((hw0 >> 8) & 0xFF)
+                cu_end = np.array([e[wg_cu == c].max() for c in np.unique(wg_cu)])
+                print(f"  compute units by the end of their last workgroup: min {cu_end.min():.2f}, median "
+                      f"{np.median(cu_end):.2f}, 90th percentile {np.percentile(cu_end, 90):.2f}, max {cu_end.max():.2f}")
+                shape = dict(kv.split("=") for kv in capi.describe_launch("vec", 4, 1, 1, K, S, g).split() if "=" in kv
+                             and kv.split("=")[0] in ("strips", "splits"))
+                strips, splits = int(shape["strips"]), int(shape["splits"])
+                if splits * strips == wgs and splits > 1:
+                    sp = idx // strips
+                    print("  by split: " + "  ".join(f"{k}: {np.median(e[sp == k]):.2f} / {e[sp == k].max():.2f}"
+                                                     for k in range(splits)))
     finally:
         capi.tune(9, 0)
     acc = np.array(acc).mean(axis=0)
