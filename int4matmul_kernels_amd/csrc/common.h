@@ -69,6 +69,23 @@ __device__ __forceinline__ h16 dequant_code(uint32_t q, h16 scale, h16 zero) {
     return __builtin_fmaf16((h16)(float)iv, -scale, zero);
 }
 
+// Exponent quantisation on magic-number operands.  A magic-number pair {2^a | q << o, 2^b | q' << o'}
+// holds its two codes inside the mantissas, at offsets o, o' with 2^(10 - o) = 2^a the half's magic
+// offset; a packed 16-bit multiply by those offsets (`offsets` = 2^a | 2^b << 16, as integers)
+// moves both codes to bits 10.. of their halves -- whatever the magic bits turn into lies above
+// the code and is masked away.  The code's low BITS - 1 bits are then the exponent field's
+// increment over 15 (2^0) and its top bit is the sign: the half becomes +-2^(code's low bits),
+// the value the exponent mode multiplies by (matmul.cuh:127-136).
+typedef uint16_t u16x2 __attribute__((ext_vector_type(2)));
+template <int BITS>
+__device__ __forceinline__ uint32_t expo_operand(uint32_t h, uint32_t offsets) {
+    const uint32_t m = bitcast<uint32_t>(bitcast<u16x2>(h) * bitcast<u16x2>(offsets));
+    constexpr uint32_t E1 = ((1u << (BITS - 1)) - 1u) << 10, EMASK = E1 | (E1 << 16);
+    const uint32_t magnitude = (m & EMASK) + 0x3C003C00u;
+    return ((m << (6 - BITS)) & 0x80008000u) | magnitude;
+}
+__host__ __device__ constexpr uint32_t off2(uint32_t lo, uint32_t hi) { return lo | (hi << 16); }
+
 // value a code stands for before scale/zero are applied: q in linear mode,
 // +-2^(low bits) in exponent mode
 template <int BITS>

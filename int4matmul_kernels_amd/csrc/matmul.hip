@@ -338,14 +338,9 @@ __device__ __forceinline__ h16x8 dequant_chunk_fast(uint32_t bits, h16x2 negz, h
 // +-2^e comes from the pair's magic-number word {2^a | q_even, 2^b | q_odd << BITS}: a packed
 // 16-bit multiply moves both codes to bits 10.. of their halves (the magic bits leave through the
 // top), the low BITS - 1 bits are the exponent field's increment over 15, the top bit is the sign.
-typedef uint16_t u16x2 __attribute__((ext_vector_type(2)));
 template <int BITS>
 __device__ __forceinline__ h16x2 expo_pair(uint32_t h) {
-    const u16x2 mul = {(uint16_t)1024, (uint16_t)(1u << (10 - BITS))};
-    const uint32_t m = bitcast<uint32_t>(bitcast<u16x2>(h) * mul);
-    constexpr uint32_t E1 = ((1u << (BITS - 1)) - 1u) << 10, EMASK = E1 | (E1 << 16);
-    const uint32_t magnitude = (m & EMASK) + 0x3C003C00u;
-    return as_h2(((m << (6 - BITS)) & 0x80008000u) | magnitude);
+    return as_h2(expo_operand<BITS>(h, off2(1024u, 1u << (10 - BITS))));
 }
 
 template <int BITS>

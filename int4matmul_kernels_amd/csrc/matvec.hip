@@ -106,20 +106,6 @@ __device__ __forceinline__ uint32_t and_or(uint32_t w, uint32_t mask, uint32_t m
     return (w & mask) | magic;
 }
 
-// Exponent quantisation on the same operands.  A magic-number pair holds its two codes inside
-// the mantissas, at offsets o with 2^(10 - o) the pair's magic offsets; a packed 16-bit multiply
-// by those offsets moves both codes to bits 10.. of their halves (whatever the magic bits turn
-// into lies above and is masked away).  The code's low BITS - 1 bits are then the exponent
-// field's increment over 15 (2^0) and its top bit is the sign: the half is +-2^(code's low bits),
-// the value the exponent mode multiplies by (matmul.cuh:127-136).
-typedef uint16_t u16x2 __attribute__((ext_vector_type(2)));
-template <int BITS>
-__device__ __forceinline__ uint32_t expo_operand(uint32_t h, uint32_t offsets) {
-    const uint32_t m = bitcast<uint32_t>(bitcast<u16x2>(h) * bitcast<u16x2>(offsets));
-    constexpr uint32_t E1 = ((1u << (BITS - 1)) - 1u) << 10, EMASK = E1 | (E1 << 16);
-    const uint32_t magnitude = (m & EMASK) + 0x3C003C00u;
-    return ((m << (6 - BITS)) & 0x80008000u) | magnitude;
-}
 // operand of the matrix core for one pair: {2^a + q, 2^b + q'} (linear mode, offsets removed
 // later) or {+-2^e, +-2^e'} (exponent mode, nothing to remove); `offsets` = {2^a, 2^b} as integers
 template <int BITS, bool EXPO>
@@ -128,7 +114,6 @@ __device__ __forceinline__ uint32_t operand(uint32_t w, uint32_t mask, uint32_t 
     if constexpr (EXPO) return expo_operand<BITS>(h, offsets);
     else return h;
 }
-__host__ __device__ constexpr uint32_t off2(uint32_t lo, uint32_t hi) { return lo | (hi << 16); }
 
 // ---- fast paths.  xp points at the unit's staged states (LDS).
 //

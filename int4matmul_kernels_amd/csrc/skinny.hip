@@ -158,13 +158,30 @@ __device__ __forceinline__ h16x8 exact_operand_sparse(uint32_t v, uint32_t m8, h
     return o;
 }
 
+// The chunk's 8 fp16 weights themselves, in the operand's k order, in either quantisation mode
+// (the mode belongs to the lane's column and group), bit-exact with dequant_code and without a
+// branch: from the magic-number pairs, P = the codes (offsets removed, exact) or +-2^e,
+//     A = P + N (one rounding),  w = fma(A, B, C) (one rounding)
+// with (N, B, C) = (-z, s, -0) for a linear group -- fp16(q - z), then fp16(. * s); adding -0
+// changes no bit -- and (-0, -s, z) for an exponent group, the reference's single-rounded fma.
 template <int BITS>
-__device__ __forceinline__ h16x8 exact_operand(uint32_t f, h16 sc, h16 ze) {
-    h16x8 r;
+__device__ __forceinline__ h16x8 exact_operand(uint32_t f, uint32_t m0, uint32_t m1, uint32_t g0, uint32_t g1,
+                                               h16 sc, h16 ze) {
+    const u32x4 h = bitcast<u32x4>(magic_operand<BITS>(f, m0, m1, g0, g1));
+    const bool expo = !(sc >= (h16)0.0f);
+    const h16x2 minus0 = as_h2(0x80008000u), s2 = {sc, sc}, z2 = {ze, ze};
+    const h16x2 N = expo ? minus0 : -z2, B = expo ? -s2 : s2, C = expo ? z2 : minus0;
+    u32x4 r;
 #pragma unroll
-    for (int e = 0; e < 8; ++e)
-        r[e] = dequant_code<BITS>((f >> (BITS * SkFmt<BITS>::order(e))) & ((1u << BITS) - 1u), sc, ze);
-    return r;
+    for (int e = 0; e < 4; ++e) {
+        const uint32_t offs = SkFmt<BITS>::offs(e);                    // {2^a, 2^b} as halves
+        const h16x2 q = as_h2(h[e]) - as_h2(offs);                     // exact
+        // the same offsets as integers, for the packed multiply: 2^(exponent field - 15)
+        const uint32_t ints = off2(1u << (((offs >> 10) & 31u) - 15u), 1u << (((offs >> 26) & 31u) - 15u));
+        const h16x2 P = expo ? as_h2(expo_operand<BITS>(h[e], ints)) : q;
+        r[e] = as_u32(__builtin_elementwise_fma(P + N, B, C));
+    }
+    return bitcast<h16x8>(r);
 }
 
 // CW: columns per lane; RT: row groups of 8 that can hold real rows (R <= 8 RT);
@@ -419,7 +436,7 @@ __global__ __launch_bounds__(512) void skinny_kernel(SkinnyArgs a) {
                         }
                     } else {
                         const uint32_t f = chunk_bits(w, i, c);
-                        const h16x8 wb = general ? exact_operand<BITS>(f, sc[c], ze[c])
+                        const h16x8 wb = general ? exact_operand<BITS>(f, m0, m1, g0, g1, sc[c], ze[c])
                                                  : magic_operand<BITS>(f, m0, m1, g0, g1);
 #pragma unroll
                         for (int mt = 0; mt < MT; ++mt)
@@ -784,7 +801,7 @@ __global__ __launch_bounds__(512) void wide_rows_kernel(SkinnyArgs a) {
                         wb = general ? exact_operand_sparse(v, mb4 & 0xFFu, sc[c], ze[c]) : sparse_scaled_operand(v, mb4, c);
                     } else {
                         const uint32_t f = chunk_bits(wu, i, c);
-                        wb = general ? exact_operand<BITS>(f, sc[c], ze[c]) : scaled_operand(f, c);
+                        wb = general ? exact_operand<BITS>(f, m0, m1, g0, g1, sc[c], ze[c]) : scaled_operand(f, c);
                     }
 #pragma unroll
                     for (int mt = 0; mt < MT; ++mt)
