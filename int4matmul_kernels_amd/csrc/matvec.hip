@@ -825,16 +825,26 @@ static int matvec_impl(int bits, void* outs, const void* matrix, const void* mul
         if (upwg < 4) upwg = 4;
     }
     if (upwg > units_total) upwg = units_total;
-    // 160 strips x 4 splits = 640 workgroups of 4 waves leave the 256 compute units with 2 or 3
-    // workgroups each; twice the splits with half the waves are exactly 5 per compute unit, and
-    // the dense int4 kernel gains 1 - 7 % from that (measured for K = 4096 ... 11008 at S = 20480;
-    // int3 / int2 and the strips of 64 columns lose 2 - 4 %, so they keep the wider workgroups)
-    if (tuning(TUNE_MV_WAVES) <= 0 && tuning(TUNE_MV_UNITS) <= 0 && bits == 4 && sparse_mask == nullptr && lk == 2) {
-        const int s1 = (units_total + upwg - 1) / upwg, half = (upwg + 1) / 2;
-        const int s2 = (units_total + half - 1) / half;
-        if (half >= 8 && (strips * s1) % 256 != 0 && (strips * s2) % 256 == 0 && s2 <= MV_MAX_SPLITS) {
-            upwg = half;
-            waves = 2;
+    // The workgroup of a strip's last split sums the strip up once the others have handed
+    // their partial sums over.  With equal shares it finishes its own units last (it is
+    // dispatched last) and only then starts on the reduction and the hand-over, after the
+    // streaming has ended; with about half a share it is through both while the others still
+    // stream, and the launch ends with them.  So the other splits take U / (splits - 1/2) units
+    // each and the last one the rest (measured on MI355X: 3 - 9 % faster for every format at
+    // S = 8192 ... 28672 with 3 - 5 splits) -- unless that costs the lane groups of a launch
+    // without prefetch another round.  With more splits the idle share of the last one is
+    // missed in the streaming instead (K = 11008, S = 4096, 10 splits: 8 % slower), so they
+    // keep equal shares.
+    if (tuning(TUNE_MV_UNITS) <= 0) {
+        const int s0 = (units_total + upwg - 1) / upwg;
+        if (s0 >= 2 && s0 <= 5) {
+            const int ng = waves * lk;
+            const int w = (2 * units_total + (2 * s0 - 1) - 1) / (2 * s0 - 1);        // ceil(U / (s0 - 1/2))
+            const bool prefetching = w >= 3 * ng;
+            const bool same_rounds = (w + ng - 1) / ng == (upwg + ng - 1) / ng;
+            if (w > upwg && w <= MV_MAX_UNITS_WG && units_total - (s0 - 1) * w >= 1 &&
+                (units_total + w - 1) / w == s0 && (prefetching || same_rounds))
+                upwg = w;
         }
     }
     int splits = (units_total + upwg - 1) / upwg;

@@ -16,19 +16,20 @@ def d(*a, **kw):
 def test_matvec_configurations():
     # C1: K = S = 1024, g = 64
     assert d("vec", 4, 1, 1, 1024, 1024, 64).startswith(
-        "matvec_kernel<bits=4,dense,lane_groups=4,prefetch=0> strips=16 splits=4 waves=1 units_per_workgroup=4")
-    # C2: 1280 workgroups of two waves (five per compute unit); its transposed shape: 640 workgroups of four waves
+        "matvec_kernel<bits=4,dense,lane_groups=4,prefetch=0> strips=16 splits=4 waves=2 units_per_workgroup=5")
+    # C2: 640 workgroups of four waves; the three writing splits take 23 units each, the summing one 11.
+    # Its transposed shape has 8 splits, which share K equally
     assert d("vec", 4, 1, 1, K, S, 128).startswith(
-        "matvec_kernel<bits=4,dense,lane_groups=2,prefetch=0> strips=160 splits=8 waves=2 units_per_workgroup=10")
+        "matvec_kernel<bits=4,dense,lane_groups=2,prefetch=0> strips=160 splits=4 waves=4 units_per_workgroup=23")
     assert d("vec", 4, 1, 1, S, K, 128).startswith(
         "matvec_kernel<bits=4,dense,lane_groups=4,prefetch=0> strips=80 splits=8 waves=4 units_per_workgroup=40")
     # C4: 16:32 at K = S = 16384, g = 64
     assert d("vec", 4, 1, 1, 16384, 16384, 64, sparse=True).startswith(
-        "matvec_kernel<bits=4,16:32,lane_groups=4,prefetch=1> strips=256 splits=3 waves=4 units_per_workgroup=86")
-    # C5: int3 / int2 keep 640 workgroups of four waves
+        "matvec_kernel<bits=4,16:32,lane_groups=4,prefetch=1> strips=256 splits=3 waves=4 units_per_workgroup=103")
+    # C5: int3 / int2 take the shape of C2
     for bits in (3, 2):
         assert d("vec", bits, 1, 1, K, S, 128).startswith(
-            f"matvec_kernel<bits={bits},dense,lane_groups=2,prefetch=0> strips=160 splits=4 waves=4 units_per_workgroup=20")
+            f"matvec_kernel<bits={bits},dense,lane_groups=2,prefetch=0> strips=160 splits=4 waves=4 units_per_workgroup=23")
 
 
 @pytest.mark.parametrize("bits", [4, 3, 2])
