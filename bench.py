@@ -30,12 +30,12 @@ MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 MFMA
 
 # HBM bytes per launch of i4::matvec_kernel<4,false,2,false>, from two counter runs of this script
 # (rocprofv3 --pmc FETCH_SIZE, then WRITE_SIZE, with --calibrate-copy; commands and per-dispatch
-# readings in profiles/matvec_int4_K5120_S20480.md): FETCH_SIZE 27 902.5 KiB x 2.000 (a 256 MiB
-# copy reads 131 089.8) + WRITE_SIZE 2 280.0 KiB x 1.000 (the same copy writes 262 144.0)
-MATVEC_TRAFFIC_BYTES = 59_479_040
+# readings in profiles/matvec_int4_K5120_S20480.md): FETCH_SIZE 27 640.6 KiB x 2.000 (a 256 MiB
+# copy reads 131 089.7) + WRITE_SIZE 1 000.0 KiB x 1.000 (the same copy writes 262 144.0)
+MATVEC_TRAFFIC_BYTES = 57_631_949
 # the same for i4::matmul_kernel_pipe<4,false,4,4,true,true> at M=2048, from the same two runs
-# (profiles/matmul_int4_M2048_K5120_S20480.md): 192 769.3 KiB x 2.000 + 149 153.0 KiB x 1.000
-MATMUL_TRAFFIC_BYTES = 547_524_198
+# (profiles/matmul_int4_M2048_K5120_S20480.md): 192 782.5 KiB x 2.000 + 149 164.9 KiB x 1.000
+MATMUL_TRAFFIC_BYTES = 547_563_418
 
 
 def matvec_bytes(K, S, g, bits=4):
