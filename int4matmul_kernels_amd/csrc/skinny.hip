@@ -701,23 +701,35 @@ __global__ __launch_bounds__(512) void wide_rows_kernel(SkinnyArgs a) {
         else
             return word_of<CW>(w[blk], c) >> wshift;
     };
-    // states: thread t moves chunk t % 8 of row t / 8
+    // states: thread t moves chunk t % 8 of row t / 8 (and of row t / 8 + 64 in blocks of more than 64 rows)
+    constexpr int XP = (ROWS + 63) / 64;
+    struct XRegs { u32x4 v[XP]; };
     const int xrow = t >> 3, xchunk = t & 7;
-    const bool xstore = xrow < ROWS;
-    const h16* xsrc = a.x + (int64_t)(row0 + min(xrow, R - 1)) * a.K + xchunk * 8;
+    const h16* xsrc[XP];
+#pragma unroll
+    for (int q = 0; q < XP; ++q) xsrc[q] = a.x + (int64_t)(row0 + min(xrow + 64 * q, R - 1)) * a.K + xchunk * 8;
     // (every thread loads -- rows beyond R re-read row R - 1, their products are never written: a load
     // under a branch would make the compiler wait for all loads in flight at every use of one)
-    auto load_x = [&](int u) -> u32x4 { return *reinterpret_cast<const u32x4*>(xsrc + u * 64); };
-    auto stage_x = [&](const u32x4 v, int p) {
-        u32x4 q = v;
-        if constexpr (BITS == 4)         // the k order inside the chunk that the operand decode produces
-            q = u32x4{__builtin_amdgcn_perm(v[2], v[0], 0x05040100u), __builtin_amdgcn_perm(v[2], v[0], 0x07060302u),
-                      __builtin_amdgcn_perm(v[3], v[1], 0x05040100u), __builtin_amdgcn_perm(v[3], v[1], 0x07060302u)};
-        if (xstore) *reinterpret_cast<u32x4*>(xb + p * XBUF + xrow * SK_PITCH + xchunk * 16) = q;
+    auto load_x = [&](int u) -> XRegs {
+        XRegs r;
+#pragma unroll
+        for (int q = 0; q < XP; ++q) r.v[q] = *reinterpret_cast<const u32x4*>(xsrc[q] + u * 64);
+        return r;
+    };
+    auto stage_x = [&](const XRegs& x, int p) {
+#pragma unroll
+        for (int k = 0; k < XP; ++k) {
+            const u32x4 v = x.v[k];
+            u32x4 q = v;
+            if constexpr (BITS == 4)         // the k order inside the chunk that the operand decode produces
+                q = u32x4{__builtin_amdgcn_perm(v[2], v[0], 0x05040100u), __builtin_amdgcn_perm(v[2], v[0], 0x07060302u),
+                          __builtin_amdgcn_perm(v[3], v[1], 0x05040100u), __builtin_amdgcn_perm(v[3], v[1], 0x07060302u)};
+            if (xrow + 64 * k < ROWS) *reinterpret_cast<u32x4*>(xb + p * XBUF + (xrow + 64 * k) * SK_PITCH + xchunk * 16) = q;
+        }
     };
 
     words_t w[PF][NL];
-    u32x4 xr[PF];
+    XRegs xr[PF];
     const uint32_t m0 = vgpr_const(BITS == 4 ? 0x000F000Fu : BITS == 2 ? 0x000C0003u : 0x00380007u);
     const uint32_t g0 = vgpr_const(BITS == 4 ? 0x64006400u : BITS == 2 ? 0x5C006400u : 0x58006400u);
     const uint32_t m1 = BITS == 4 ? vgpr_const(0x00F000F0u) : 0u, g1 = BITS == 4 ? vgpr_const(0x54005400u) : 0u;
@@ -775,7 +787,7 @@ __global__ __launch_bounds__(512) void wide_rows_kernel(SkinnyArgs a) {
 #pragma unroll
     for (int f = 0; f < PF; ++f) load_w(w[f], min(u0 + f, u1 - 1));
     {
-        const u32x4 first = load_x(u0);
+        const XRegs first = load_x(u0);
 #pragma unroll
         for (int f = 0; f < PF; ++f) xr[f] = load_x(min(u0 + 1 + f, u1 - 1));
         const bool general = scan_scales();
@@ -783,7 +795,7 @@ __global__ __launch_bounds__(512) void wide_rows_kernel(SkinnyArgs a) {
         __syncthreads();
 
         // p: the LDS buffer that holds unit u; xn: the states of unit u + 1
-        auto step = [&](auto mode, int u, int p, words_t wu[NL], u32x4& xn) {
+        auto step = [&](auto mode, int u, int p, words_t wu[NL], XRegs& xn) {
             constexpr bool general = decltype(mode)::value;
             if (u == u0 || u % a.group_units == 0) load_sz(u / a.group_units);
 #pragma unroll
@@ -895,18 +907,34 @@ static WidePlan plan_wide(int64_t R, int64_t K, int64_t S, bool sparse) {
     // (knob: 1 = never, n >= 2 = from n rows on whatever the shape)
     const int64_t knob = tuning(TUNE_NO_WIDE), min_rows = knob >= 2 ? knob : 17;
     if (R < min_rows || R > SK_WIDE_MAX_ROWS || S % 256 != 0 || K % 64 != 0 || knob == 1) return p;
-    p.row_blocks = (int)((R + 63) / 64);
-    p.block_rows = (int)(((R + p.row_blocks - 1) / p.row_blocks + 15) / 16 * 16);
-    p.mt = p.block_rows / 16;
-    const int64_t wgs = S / 256 * p.row_blocks, units = K / 64;
-    // (one workgroup per CU: as many splits as keep the grid within one round of 256 -- a grid a little larger
-    // than that runs a second round -- and four when even the unsplit grid leaves a third of the CUs idle)
-    int64_t ks = 256 / wgs;
-    if (ks <= 1 && wgs > 128 && wgs < 256) ks = 4;
-    ks = std::max<int64_t>(1, std::min<int64_t>(ks, units / 8));
-    const int64_t forced = tuning(TUNE_MM_SPLIT);
-    if (forced >= 1) ks = std::min<int64_t>(forced, std::max<int64_t>(1, units / 4));
-    if (wgs > 1024) ks = 1;
+    // Row blocks of up to 64 rows, or (dense; the 16:32 decode leaves registers for 64) of up to 128: every row
+    // block decodes the strip's weights again, so two blocks of 64 rows cost nearly twice one block of 128 --
+    // unless halving the number of workgroups means splitting K more than about six ways to fill the GPU, or
+    // into shares of less than 20 units, where the hand-over of the partial tiles (twice as large, twice as
+    // many) takes the gain back (measured: K=5120, S=20480, 128 rows 70 -> 52 us, int3 76 -> 58; K=8192,
+    // S=28672, 128 rows 127 -> 95 us; K=28672, S=8192, 192 rows 172 -> 132 us; K=S=8192, 128 rows, 8 splits
+    // instead of 4: 41 -> 46 us; K=2048, S=16384, 128 rows, shares of 8 units: 25 -> 30 us)
+    const int64_t units = K / 64, forced = tuning(TUNE_MM_SPLIT);
+    int64_t wgs = 0, ks = 1;
+    auto shape = [&](int64_t tallest) {
+        p.row_blocks = (int)((R + tallest - 1) / tallest);
+        p.block_rows = (int)(((R + p.row_blocks - 1) / p.row_blocks + 15) / 16 * 16);
+        p.mt = p.block_rows / 16;
+        if (p.mt == 5) p.mt = 6;                      // (instantiated: 1, 2, 3, 4, 6, 8 tiles of 16 rows)
+        if (p.mt == 7) p.mt = 8;
+        p.block_rows = p.mt * 16;
+        wgs = S / 256 * p.row_blocks;
+        // (one workgroup per CU: as many splits as keep the grid within one round of 256 -- a grid a little
+        // larger than that runs a second round -- and four when even the unsplit grid leaves a third of the
+        // CUs idle)
+        ks = 256 / wgs;
+        if (ks <= 1 && wgs > 128 && wgs < 256) ks = 4;
+        ks = std::max<int64_t>(1, std::min<int64_t>(ks, units / 8));
+        if (forced >= 1) ks = std::min<int64_t>(forced, std::max<int64_t>(1, units / 4));
+        if (wgs > 1024) ks = 1;
+    };
+    shape(128);
+    if (sparse || R <= 64 || ks > 6 || (ks > 1 && units / ks < 20)) shape(64);
     p.units_per_split = (int)((units + ks - 1) / ks);
     p.ksplit = (int)((units + p.units_per_split - 1) / p.units_per_split);
     // measured against the kernel above (K = 2048 ... 20480, S = 1024 ... 28672): with 17 ... 32 rows it
@@ -945,7 +973,7 @@ static bool launch_wide(SkinnyArgs a, const WidePlan& p, hipStream_t st) {
                grid.x, grid.y, grid.z))
         return true;
     auto go = [&](auto kernel, int slot) {
-        static std::atomic<uint64_t> done[4];
+        static std::atomic<uint64_t> done[6];
         int dev = 0;
         hipGetDevice(&dev);
         const uint64_t bit = 1ull << (dev & 63);
@@ -958,7 +986,11 @@ static bool launch_wide(SkinnyArgs a, const WidePlan& p, hipStream_t st) {
     if (p.mt == 1) go(wide_rows_kernel<BITS, 1, SPARSE>, 0);
     else if (p.mt == 2) go(wide_rows_kernel<BITS, 2, SPARSE>, 1);
     else if (p.mt == 3) go(wide_rows_kernel<BITS, 3, SPARSE>, 2);
-    else go(wide_rows_kernel<BITS, 4, SPARSE>, 3);
+    else if (p.mt == 4) go(wide_rows_kernel<BITS, 4, SPARSE>, 3);
+    else if constexpr (!SPARSE) {
+        if (p.mt == 6) go(wide_rows_kernel<BITS, 6, SPARSE>, 4);
+        else go(wide_rows_kernel<BITS, 8, SPARSE>, 5);
+    } else return false;
     return true;
 }
 

@@ -55,6 +55,13 @@ def test_few_rows_and_batches():
     assert d("mtx", 4, 1, 8, K, S, 128).startswith("skinny_kernel<bits=4,dense,columns_per_lane=4,row_tiles=1> strips=320")
     assert d("vec", 4, 8, 1, K, S, 128).startswith("skinny_kernel<bits=4,dense,columns_per_lane=4,row_tiles=1> strips=320")
     assert d("mtx", 4, 1, 64, K, S, 128).startswith("wide_rows_kernel<bits=4,dense,row_tiles=4> strips=80 row_blocks=1 ksplit=3")
+    # 65 ... 128 rows in one block of six or eight 16-row tiles where K is split into long shares, in two blocks of
+    # four where the split would have to be deeper or shorter
+    assert d("mtx", 4, 1, 128, K, S, 128).startswith("wide_rows_kernel<bits=4,dense,row_tiles=8> strips=80 row_blocks=1 ksplit=3")
+    assert d("mtx", 3, 1, 70, K, S, 128).startswith("wide_rows_kernel<bits=3,dense,row_tiles=6> strips=80 row_blocks=1 ksplit=3")
+    assert d("mtx", 4, 1, 128, 8192, 8192, 128).startswith("wide_rows_kernel<bits=4,dense,row_tiles=4> strips=32 row_blocks=2 ksplit=4")
+    assert d("mtx", 4, 1, 128, 2048, 16384, 64).startswith("wide_rows_kernel<bits=4,dense,row_tiles=4> strips=64 row_blocks=2 ksplit=2")
+    assert d("mtx", 4, 1, 200, 28672, 8192, 128).startswith("wide_rows_kernel<bits=4,dense,row_tiles=8> strips=32 row_blocks=2 ksplit=4")
     assert d("mtx", 4, 1, 16, S, K, 128).startswith("skinny_kernel<bits=4,dense")
     assert d("mtx", 4, 1, 257, K, S, 128).startswith("matmul_kernel_pipe<bits=4,dense,tile=128x256")
 

@@ -342,3 +342,45 @@ def test_shared_staging_sparse_default_rule(H, M):
     """K=4096, S=8192 (32 M weights), 16:32: 33 rows and more take the shared-staging kernel by default"""
     p = O.make_problem(bits=4, K=4096, S=8192, M=M, group_size=64, sparse=True, seed=M)
     _check(H, p, "mtx")
+
+
+# ---- row blocks of 96 / 128 rows (dense formats): one workgroup keeps up to eight 16-row tiles per column pair
+# and stages two rows of states per thread.  Taken where K is not split at all or split into long shares.
+@pytest.mark.parametrize("bits", [4, 3, 2])
+@pytest.mark.parametrize("M,K,S,g", [(100, 512, 512, 64), (128, 512, 256, 128), (70, 320, 1024, 64), (65, 448, 256, -1),
+                                     (256, 512, 512, 128), (129, 512, 256, 64), (200, 256, 768, 64)])
+def test_tall_row_blocks(H, bits, M, K, S, g):
+    tiles = H.capi.describe_launch("mtx", bits, 1, M, K, S, g)
+    assert "wide_rows_kernel" in tiles and ("row_tiles=6" in tiles or "row_tiles=8" in tiles), tiles
+    p = _problem(bits, K=K, S=S, M=M, group_size=g, seed=M + K + S)
+    d = H.dev_problem(p)
+    exact, f32 = H.oracles(p)
+    got = H.run_capi(p, d, "mtx", outs_init=np.full((1, M, S), 2.0, np.float16))
+    H.assert_product_close(got, exact, f32, kind="mtx")
+    again = H.run_capi(p, d, "mtx")
+    assert np.array_equal(got, again)
+    H.capi.tune(8, 1)                          # the kernel whose waves stage their own states
+    try:
+        ref = H.run_capi(p, d, "mtx")
+    finally:
+        H.capi.tune(8, 0)
+    assert O.max_rel_error(ref.astype(np.float64), got) < H.TOL_EXACT_MTX
+
+
+@pytest.mark.parametrize("bits", [4, 3, 2])
+def test_tall_row_blocks_exponent_mode_and_batches(H, bits):
+    """exponent-mode columns take the general decode of the same kernel; batches flatten into rows"""
+    p = _problem(bits, K=512, S=512, M=25, B=5, group_size=128, seed=31)
+    assert "row_tiles=8" in H.capi.describe_launch("mtx", bits, 5, 25, 512, 512, 128)
+    p["scales"][1, 40:48] *= np.float16(-1)
+    p["scales"][3, 300] *= np.float16(-1)
+    _check(H, p, "mtx")
+
+
+@pytest.mark.parametrize("bits,M", [(4, 128), (4, 70), (3, 128), (2, 96)])
+def test_tall_row_blocks_full_size_split_k(H, bits, M):
+    """K=5120, S=20480: 80 strips, K split three ways, partial tiles of 96 / 128 rows handed over"""
+    tiles = H.capi.describe_launch("mtx", bits, 1, M, 5120, 20480, 128)
+    assert "row_blocks=1 ksplit=3" in tiles and ("row_tiles=6" in tiles or "row_tiles=8" in tiles), tiles
+    p = _problem(bits, K=5120, S=20480, M=M, group_size=128, seed=M)
+    _check(H, p, "mtx")
