@@ -1108,12 +1108,14 @@ bool skinny_rows(int bits, h16* outs, const uint32_t* matrix, const h16* x, cons
         }
     }
     if (R > 96) return false;
-    // four waves split K when there are 256 workgroups (three of them fit a CU) and K
-    // is short (each wave should walk a dozen units or more), eight otherwise
+    // four waves split K when there are more workgroups than CUs (three of them fit a CU) and K
+    // is short (each wave should walk a dozen units or more), eight otherwise -- also at exactly one
+    // workgroup per CU, where eight waves keep twice the bytes in flight (K=5120, S=16384, 8 rows:
+    // 14.6 -> 12.0 us; K=S=8192: 16.5 -> 12.3 us; 320 and 448 strips: 17.7 against 22.2, 27 against 32)
     int cw = unsplit_cw(R, S, sparse_mask != nullptr);
     const int units = (int)(K / 64);
     int waves = (int)tuning(TUNE_MV_WAVES);
-    if (waves != 2 && waves != 4 && waves != 8) waves = S / (16 * cw) >= 256 && units < 160 ? 4 : 8;
+    if (waves != 2 && waves != 4 && waves != 8) waves = S / (16 * cw) > 256 && units < 160 ? 4 : 8;
     while (waves > 1 && units < 2 * waves) waves >>= 1;
     auto launch = [&](int cw_, int waves_, int ksplit_) {
         a.units_per_wave = (a.units_per_split + waves_ - 1) / waves_;
