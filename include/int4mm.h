@@ -81,8 +81,9 @@ INT4MM_API int int4mm_abi_version(void);
  * workgroup of the matvec and few-row kernels, 1 = matvec 64-row units per lane
  * group, 2 = matvec lane groups per wave (1, 2, 4), 3 = matmul kernel variant
  * (5 / 6 / 7 = pipelined 256x128 / 256x256 / 128x256 tiles, 9 = 256x256 without
- * the two-phase order), 4 = matvec: 1 disables prefetch,
- * 5 = 1 disables the few-row (2..256 rows) kernels, 6 = split-K factor of the
+ * the two-phase order; a forced variant also keeps the product away from the
+ * few-row kernels), 4 = matvec: 1 disables prefetch,
+ * 5 = 1 disables the few-row (2..512 rows) kernels, 6 = split-K factor of the
  * matmul and few-row kernels (1 = never split, 2..8 = that factor where the
  * shape allows a split at all), 7 = 1: the tiles of a matmul's last, partly
  * filled round are not split, 8 = the few-row kernel whose waves share the

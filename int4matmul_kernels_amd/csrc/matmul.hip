@@ -1200,8 +1200,9 @@ extern "C" int int4mm_matmul(int bits, void* outs, const void* matrix, const voi
     const int64_t g = shape->group_size < 0 ? ONE_GROUP : shape->group_size;
 
     hipStream_t st = (hipStream_t)stream;
-    // 2 .. 96 rows in all (batches are contiguous, so they flatten): the HBM-bound few-row kernel
-    if (B * M >= 2 && B * M <= SK_WIDE_MAX_ROWS && !tuning(TUNE_NO_SKINNY) &&
+    // 2 .. 96 rows in all (batches are contiguous, so they flatten; on suitable shapes up to 512): the few-row
+    // kernels, which read every packed word once for all rows -- unless a tile-kernel variant is forced
+    if (B * M >= 2 && B * M <= SK_WIDE_MAX_ROWS && !tuning(TUNE_NO_SKINNY) && !tuning(TUNE_MM_VARIANT) &&
         skinny_rows(bits, (h16*)outs, (const uint32_t*)matrix, (const h16*)multiplier, (const h16*)scales,
                     (const h16*)zeros, B * M, K, S, g, false, st, (const uint32_t*)sparse_mask, workspace, workspace_bytes))
         return check_launch("matmul");

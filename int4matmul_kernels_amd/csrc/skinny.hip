@@ -596,7 +596,7 @@ __global__ __launch_bounds__(512) void skinny_kernel(SkinnyArgs a) {
     }
 }
 
-// ---- 17 ... 256 rows, every format: the eight waves of a workgroup share one staged copy of the states.
+// ---- 17 ... 512 rows, every format: the eight waves of a workgroup share one staged copy of the states.
 // In the kernel above every wave stages the states of its own units, so a workgroup of 64 columns reads
 // all R x K states: with R = 64 that is four times the packed weights it reads.  Here the waves stand side
 // by side along the columns (32 each, 256 per workgroup), all walk the same units, and each unit's states
@@ -902,7 +902,20 @@ __global__ __launch_bounds__(512) void wide_rows_kernel(SkinnyArgs a) {
 // Plan of the wide kernel: row blocks of 16 ... 64 rows, 256-column strips, K split over about as many
 // workgroups as there are CUs (at least 8 units each; one counter per strip and row block: at most 1024).
 struct WidePlan { bool use; int mt, row_blocks, block_rows, ksplit, units_per_split; size_t part_bytes; };
-static WidePlan plan_wide(int64_t R, int64_t K, int64_t S, bool sparse) {
+// LDS of the wide kernel: two unit buffers of states, a flag, the selector table's alignment slack, and the
+// strip's scales and zeros for the workgroup's share of K (1 KB per quantisation group)
+static size_t wide_lds_bytes(int block_rows, int64_t groups) {
+    return 2 * (size_t)block_rows * SK_PITCH + 1024 + 16 + (size_t)groups * 256 * 4;
+}
+static int64_t wide_groups(int64_t units, int64_t units_per_split, int64_t ksplit, int64_t group_units) {
+    int64_t groups = (units + group_units - 1) / group_units;
+    if (ksplit > 1) groups = std::min(groups, (units_per_split + group_units - 1) / group_units + 1);
+    return groups;
+}
+constexpr size_t WIDE_LDS_LIMIT = 150 * 1024;
+
+// `group_units`: 64-row units per quantisation group (K / 64 and more: a single group)
+static WidePlan plan_wide(int64_t R, int64_t K, int64_t S, bool sparse, int64_t group_units) {
     WidePlan p{false, 0, 0, 0, 1, 0, 0};
     // (knob: 1 = never, n >= 2 = from n rows on whatever the shape)
     const int64_t knob = tuning(TUNE_NO_WIDE), min_rows = knob >= 2 ? knob : 17;
@@ -932,11 +945,20 @@ static WidePlan plan_wide(int64_t R, int64_t K, int64_t S, bool sparse) {
         ks = std::max<int64_t>(1, std::min<int64_t>(ks, units / 8));
         if (forced >= 1) ks = std::min<int64_t>(forced, std::max<int64_t>(1, units / 4));
         if (wgs > 1024) ks = 1;
+        // (a long share of K with small groups: more splits, within one round of workgroups, until the share's
+        // scales and zeros fit the LDS)
+        const size_t room = WIDE_LDS_LIMIT - (sparse ? 4096 : 0);
+        while (wgs * (ks + 1) <= 256 && ks < units / 8 &&
+               wide_lds_bytes(p.block_rows, wide_groups(units, (units + ks - 1) / ks, ks, group_units)) > room)
+            ++ks;
     };
     shape(128);
     if (sparse || R <= 64 || ks > 6 || (ks > 1 && units / ks < 20)) shape(64);
     p.units_per_split = (int)((units + ks - 1) / ks);
     p.ksplit = (int)((units + p.units_per_split - 1) / p.units_per_split);
+    if (wide_lds_bytes(p.block_rows, wide_groups(units, p.units_per_split, p.ksplit, group_units)) >
+        WIDE_LDS_LIMIT - (sparse ? 4096 : 0))
+        return p;
     // measured against the kernel above (K = 2048 ... 20480, S = 1024 ... 28672): with 17 ... 32 rows it
     // needs 32 ... 96 strips and long shares of K, with 33 ... 64 rows matrices of 32 M weights and more
     // and from 129 rows on the tile kernels win on wide outputs
@@ -961,11 +983,8 @@ static WidePlan plan_wide(int64_t R, int64_t K, int64_t S, bool sparse) {
 
 template <int BITS, bool SPARSE = false>
 static bool launch_wide(SkinnyArgs a, const WidePlan& p, hipStream_t st) {
-    const int upg = a.group_units;
-    int groups = (a.K / 64 + upg - 1) / upg;
-    if (p.ksplit > 1) groups = std::min(groups, (p.units_per_split + upg - 1) / upg + 1);
-    const size_t lds = 2 * (size_t)p.block_rows * SK_PITCH + 1024 + 16 + (size_t)groups * 256 * 4;
-    if (lds > 150 * 1024 - (SPARSE ? 4096 : 0)) return false;
+    const size_t lds = wide_lds_bytes(p.block_rows, wide_groups(a.K / 64, p.units_per_split, p.ksplit, a.group_units));
+    if (lds > WIDE_LDS_LIMIT - (SPARSE ? 4096 : 0)) return false;
     a.block_rows = p.block_rows;
     a.units_per_split = p.units_per_split;
     const dim3 grid((unsigned)(a.S / 256), (unsigned)p.row_blocks, (unsigned)p.ksplit), block(512);
@@ -1073,8 +1092,10 @@ static SkinnySplit plan_skinny_split(int64_t R, int64_t K, int64_t S, bool spars
 
 size_t skinny_workspace_bytes(int64_t R, int64_t K, int64_t S, bool sparse) {
     const SkinnySplit p = plan_skinny_split(R, K, S, sparse);
-    const WidePlan wp = plan_wide(R, K, S, sparse);
-    return std::max<size_t>(p.ksplit > 1 ? p.part_bytes : 0, wp.use ? wp.part_bytes : 0);
+    // (the split of the wide kernel can depend on the group size: room for the smallest groups and for one)
+    const WidePlan w1 = plan_wide(R, K, S, sparse, 1), wn = plan_wide(R, K, S, sparse, 0x7FFFFFF);
+    const size_t wide = std::max<size_t>(w1.use ? w1.part_bytes : 0, wn.use ? wn.part_bytes : 0);
+    return std::max<size_t>(p.ksplit > 1 ? p.part_bytes : 0, wide);
 }
 
 // Product of 2 <= R <= 96 rows with a dense or (sparse_mask != nullptr) 16:32 sparse int4 matrix; beyond that
@@ -1096,7 +1117,7 @@ bool skinny_rows(int bits, h16* outs, const uint32_t* matrix, const h16* x, cons
     a.counters = nullptr;
     // 33 rows and more, dense: the kernel whose waves share the staged states
     {
-        const WidePlan wp = plan_wide(R, K, S, sparse_mask != nullptr);
+        const WidePlan wp = plan_wide(R, K, S, sparse_mask != nullptr, a.group_units);
         const WorkspaceParts ws = workspace_parts(workspace, workspace_bytes);
         if (wp.use && (wp.ksplit == 1 || (ws.counters != nullptr && ws.scratch_bytes >= wp.part_bytes))) {
             a.units_per_wave = 0;

@@ -5,7 +5,7 @@ dequantises its weights returns them unchanged: the fp32 sum of 1 * w and zeros 
 w, and rounding it to fp16 gives back the fp16 weight.  So ``outs`` must equal the
 oracle's dequantised matrix (oracle.dequantize_matrix, the restatement of
 matmul.cuh:115-136,246-428) BIT FOR BIT -- for every tile kernel variant, the
-few-row kernel that dequantises (17 .. 256 rows), with and without split-K, all four
+few-row kernel that dequantises (17 .. 512 rows), with and without split-K, all four
 formats, linear and exponent-mode groups.  (Zero weights are compared by value: a
 sum of +0.0 and -0.0 is +0.0.)  The matvec and the 2 .. 16 row kernel apply scale
 and zero per group in fp32 instead of dequantising, so they are not subject to

@@ -1,4 +1,4 @@
-"""The few-row kernels (2 .. 96 rows of states in all, dense formats on suitable shapes up to 256; dense
+"""The few-row kernels (2 .. 96 rows of states in all, on suitable shapes up to 512; dense
 formats and 16:32 sparse int4): every packed word is read once for all rows.  It serves `quant_matmul` with small M (any
 batch layout that flattens to <= 32 rows) and the matvec entry with B > 1.
 Its numerics are the matvec's (exact sum of x (q - z) s, no per-weight fp16
@@ -256,10 +256,12 @@ def test_shared_staging_rows_default_rule_large_matrix(H, M):
 
 @pytest.mark.parametrize("bits", [4, 3, 2])
 @pytest.mark.parametrize("M,K,S,g", [(97, 1024, 512, 128), (128, 4096, 256, 64), (130, 2048, 768, -1), (200, 1024, 1024, 64),
-                                     (256, 2048, 512, 128), (129, 320, 256, 64)])
-def test_shared_staging_up_to_256_rows(H, bits, M, K, S, g):
-    """97 ... 256 rows (up to four row blocks of 64): the weights are dequantised with the reference's two
+                                     (256, 2048, 512, 128), (129, 320, 256, 64), (257, 1024, 512, 64), (300, 2048, 256, 128),
+                                     (384, 512, 768, 64), (449, 1536, 256, -1), (512, 1024, 512, 128)])
+def test_shared_staging_up_to_512_rows(H, bits, M, K, S, g):
+    """97 ... 512 rows (row blocks of up to 64 or 128 rows): the weights are dequantised with the reference's two
     roundings, so the matmul tolerance against the product on fp16 weights holds"""
+    assert "wide_rows_kernel" in H.capi.describe_launch("mtx", bits, 1, M, K, S, g)
     p = _problem(bits, K=K, S=S, M=M, group_size=g, seed=M + K + S)
     d = H.dev_problem(p)
     exact, f32 = H.oracles(p)

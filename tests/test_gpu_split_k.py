@@ -16,7 +16,7 @@ from oracle import oracle as O  # noqa: E402
 @pytest.fixture(scope="module")
 def H():
     from tests import helpers
-    helpers.capi.tune(8, 1)          # (up to 256 rows would otherwise take the few-row path: not the subject here)
+    helpers.capi.tune(8, 1)          # (up to 512 rows would otherwise take the few-row path: not the subject here)
     yield helpers
     helpers.capi.tune(8, 0)
 
