@@ -610,7 +610,8 @@ __global__ __launch_bounds__(512) void skinny_kernel(SkinnyArgs a) {
 template <int BITS, int MT, bool SPARSE = false>
 __global__ __launch_bounds__(512) void wide_rows_kernel(SkinnyArgs a) {
     using F = SkFmt<BITS, SPARSE>;
-    constexpr int CW = 2, NL = F::LOADS, PF = 4, ROWS = 16 * MT, STRIP = 16 * CW, WSTRIP = 8 * STRIP;
+    // (units of weights in flight per wave: four; two in the tall 16:32 blocks, whose registers are short)
+    constexpr int CW = 2, NL = F::LOADS, PF = (SPARSE && MT > 4) ? 2 : 4, ROWS = 16 * MT, STRIP = 16 * CW, WSTRIP = 8 * STRIP;
     constexpr int XBUF = ROWS * SK_PITCH;
     extern __shared__ __attribute__((aligned(16))) char lds[];
     typedef typename Words<CW>::type words_t;
@@ -920,13 +921,15 @@ static WidePlan plan_wide(int64_t R, int64_t K, int64_t S, bool sparse, int64_t 
     // (knob: 1 = never, n >= 2 = from n rows on whatever the shape)
     const int64_t knob = tuning(TUNE_NO_WIDE), min_rows = knob >= 2 ? knob : 17;
     if (R < min_rows || R > SK_WIDE_MAX_ROWS || S % 256 != 0 || K % 64 != 0 || knob == 1) return p;
-    // Row blocks of up to 64 rows, or (dense; the 16:32 decode leaves registers for 64) of up to 128: every row
-    // block decodes the strip's weights again, so two blocks of 64 rows cost nearly twice one block of 128 --
+    // Row blocks of up to 64 rows, or of up to 128 (16:32: with two units of weights in flight per wave instead
+    // of four, for the registers): every row block decodes the strip's weights again, so two blocks of 64 rows
+    // cost nearly twice one block of 128 --
     // unless halving the number of workgroups means splitting K more than about six ways to fill the GPU, or
     // into shares of less than 20 units, where the hand-over of the partial tiles (twice as large, twice as
     // many) takes the gain back (measured: K=5120, S=20480, 128 rows 70 -> 52 us, int3 76 -> 58; K=8192,
     // S=28672, 128 rows 127 -> 95 us; K=28672, S=8192, 192 rows 172 -> 132 us; K=S=8192, 128 rows, 8 splits
-    // instead of 4: 41 -> 46 us; K=2048, S=16384, 128 rows, shares of 8 units: 25 -> 30 us)
+    // instead of 4: 41 -> 46 us; K=2048, S=16384, 128 rows, shares of 8 units: 25 -> 30 us; 16:32, K=5120,
+    // S=20480: 96 rows 92 -> 51 us, 128 rows 79 (256-row tiles) -> 60 us)
     const int64_t units = K / 64, forced = tuning(TUNE_MM_SPLIT);
     int64_t wgs = 0, ks = 1;
     auto shape = [&](int64_t tallest) {
@@ -953,7 +956,7 @@ static WidePlan plan_wide(int64_t R, int64_t K, int64_t S, bool sparse, int64_t 
             ++ks;
     };
     shape(128);
-    if (sparse || R <= 64 || ks > 6 || (ks > 1 && units / ks < 20)) shape(64);
+    if (R <= 64 || ks > 6 || (ks > 1 && units / ks < 20)) shape(64);
     p.units_per_split = (int)((units + ks - 1) / ks);
     p.ksplit = (int)((units + p.units_per_split - 1) / p.units_per_split);
     if (wide_lds_bytes(p.block_rows, wide_groups(units, p.units_per_split, p.ksplit, group_units)) >
@@ -968,7 +971,8 @@ static WidePlan plan_wide(int64_t R, int64_t K, int64_t S, bool sparse, int64_t 
         if (sparse) {
             if (R <= 32 && K * S < (1ll << 26)) return p;
             if (R > 32 && R <= 64 && K * S < (1ll << 25)) return p;
-            if (R > 96 && R <= 128 && S > 16384) return p;       // (the padded 256-row tiles win on very wide outputs)
+            // (the padded 256-row tiles win on very wide outputs against two row blocks)
+            if (R > 96 && R <= 128 && S > 16384 && p.row_blocks > 1) return p;
             if (R > 128 && (S > 5120 || (R > 192 && S > 4096))) return p;
         } else {
             if (R <= 32 && (wgs < 32 || wgs > 96 || p.units_per_split < 16)) return p;
@@ -1006,10 +1010,8 @@ static bool launch_wide(SkinnyArgs a, const WidePlan& p, hipStream_t st) {
     else if (p.mt == 2) go(wide_rows_kernel<BITS, 2, SPARSE>, 1);
     else if (p.mt == 3) go(wide_rows_kernel<BITS, 3, SPARSE>, 2);
     else if (p.mt == 4) go(wide_rows_kernel<BITS, 4, SPARSE>, 3);
-    else if constexpr (!SPARSE) {
-        if (p.mt == 6) go(wide_rows_kernel<BITS, 6, SPARSE>, 4);
-        else go(wide_rows_kernel<BITS, 8, SPARSE>, 5);
-    } else return false;
+    else if (p.mt == 6) go(wide_rows_kernel<BITS, 6, SPARSE>, 4);
+    else go(wide_rows_kernel<BITS, 8, SPARSE>, 5);
     return true;
 }
 

@@ -386,3 +386,32 @@ def test_tall_row_blocks_full_size_split_k(H, bits, M):
     assert "row_blocks=1 ksplit=3" in tiles and ("row_tiles=6" in tiles or "row_tiles=8" in tiles), tiles
     p = _problem(bits, K=5120, S=20480, M=M, group_size=128, seed=M)
     _check(H, p, "mtx")
+
+
+@pytest.mark.parametrize("M,K,S,g", [(100, 512, 512, 64), (128, 512, 256, 128), (70, 320, 1024, 64), (96, 448, 256, -1),
+                                     (200, 512, 512, 64)])
+def test_tall_row_blocks_sparse(H, M, K, S, g):
+    """16:32 in row blocks of 96 / 128 rows (two units of weights in flight per wave)"""
+    tiles = H.capi.describe_launch("mtx", 4, 1, M, K, S, g, sparse=True)
+    assert "wide_rows_kernel<bits=4,16:32" in tiles and ("row_tiles=6" in tiles or "row_tiles=8" in tiles), tiles
+    p = O.make_problem(bits=4, K=K, S=S, M=M, group_size=g, sparse=True, seed=M + K + S)
+    p["scales"].reshape(-1, S)[-1, 8:12] *= np.float16(-1)            # a few exponent-mode columns
+    d = H.dev_problem(p)
+    exact, f32 = H.oracles(p)
+    got = H.run_capi(p, d, "mtx", outs_init=np.full((1, M, S), 2.0, np.float16))
+    H.assert_product_close(got, exact, f32, kind="mtx")
+    assert np.array_equal(got, H.run_capi(p, d, "mtx"))
+    H.capi.tune(8, 1)
+    try:
+        ref = H.run_capi(p, d, "mtx")
+    finally:
+        H.capi.tune(8, 0)
+    assert O.max_rel_error(ref.astype(np.float64), got) < H.TOL_EXACT_MTX
+
+
+def test_tall_row_blocks_sparse_full_size_split_k(H):
+    """K=5120, S=20480, g=64, 128 rows: one block of eight tiles, K split three ways"""
+    tiles = H.capi.describe_launch("mtx", 4, 1, 128, 5120, 20480, 64, sparse=True)
+    assert "wide_rows_kernel<bits=4,16:32,row_tiles=8> strips=80 row_blocks=1 ksplit=3" in tiles, tiles
+    p = O.make_problem(bits=4, K=5120, S=20480, M=128, group_size=64, sparse=True, seed=9)
+    _check(H, p, "mtx")
