@@ -1149,7 +1149,17 @@ static void launch(MatmulArgs a, int64_t B, hipStream_t st, void* workspace, siz
         const bool small_better = tiles4 <= 128 || (!tail_ok && tiles4 > 256 && tiles4 < 512 && last > 0 && last <= 96);
         // (a grid that fills at most half of the GPU with a short K: the pipelined kernel's prologue -- three
         // stages, the scan of the scales -- costs more than its faster steps return; measured K <= 1024)
+        // (a long K on a narrow output: 256 x 128 tiles split three ways and more along K, in shares of at least
+        // 140 steps, beat one round of unsplit 128 x 256 tiles -- K=20480, S=5120: 769 rows 283 -> 240 us, 1024 rows
+        // 279 -> 252 us; K=14336, S=4096, 1280 rows 198 -> 187 us; shorter shares lose: K=S=8192, 1024 rows 147 / 159)
+        bool long_k_split = false;
+        if (!SPARSE && three_rows && pipe2_ok) {
+            const SplitPlan sp = plan_split(false, B, a.M, a.K, a.S);
+            long_k_split = sp.ksplit >= 3 && a.K / 32 / sp.ksplit >= 140 && wsp.counters != nullptr &&
+                           wsp.scratch_bytes >= (size_t)(sp.tiles * sp.ksplit * sp.tile_bytes);
+        }
         if (!SPARSE && tiles4 <= 128 && a.K <= 1024) variant = 1;
+        else if (long_k_split) variant = 5;
         else if (three_rows) variant = 7;
         else if (pipe4_ok && (SPARSE || !pipe2_ok || !small_better)) variant = 6;
         else if (pipe2_ok) variant = 5;

@@ -51,6 +51,15 @@ def test_other_matmul_configurations():
         "matmul_kernel_pipe<bits=4,16:32,tile=256x256,plain> tiles=640 ksplit=2 split_from=512 workgroups=768")
 
 
+def test_long_k_on_a_narrow_output():
+    # one round of unsplit 128 x 256 tiles loses to 256 x 128 tiles split three ways when the shares of K stay long
+    assert d("mtx", 4, 1, 1024, S, K, 128).startswith("matmul_kernel_pipe<bits=4,dense,tile=256x128,plain> tiles=160 ksplit=3")
+    assert d("mtx", 4, 1, 1280, S, K, 128).startswith("matmul_kernel_pipe<bits=4,dense,tile=128x256,plain> tiles=200 ksplit=1")
+    assert d("mtx", 4, 1, 1024, 8192, 8192, 128).startswith("matmul_kernel_pipe<bits=4,dense,tile=128x256,plain> tiles=256 ksplit=1")
+    # (without a workspace for the partial tiles: unsplit)
+    assert "tile=128x256" in d("mtx", 4, 1, 1024, S, K, 128, workspace_bytes=0)
+
+
 def test_few_rows_and_batches():
     assert d("mtx", 4, 1, 8, K, S, 128).startswith("skinny_kernel<bits=4,dense,columns_per_lane=4,row_tiles=1> strips=320")
     assert d("vec", 4, 8, 1, K, S, 128).startswith("skinny_kernel<bits=4,dense,columns_per_lane=4,row_tiles=1> strips=320")

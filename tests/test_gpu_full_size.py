@@ -162,3 +162,26 @@ def test_mixed_quantisation_modes_matvec_full_size(H, bits):
         exact[:, cols] = O.matmul_exact(x, w16)
     exact = exact.reshape(1, 1, S)
     H.assert_product_close(got, exact, exact.astype(np.float32))
+
+
+@pytest.mark.parametrize("bits", [4, 3])
+def test_long_k_narrow_output_takes_split_small_tiles(H, bits):
+    """K=14336, S=4096, 1152 rows: nine rows of 128 x 256 tiles would fill the GPU once; the long K makes
+    256 x 128 tiles split three ways along K the faster choice.  Sampled rows against the oracle, the whole
+    output against the unsplit kernel."""
+    K, S, g, M = 14336, 4096, 128, 1152
+    tiles = H.capi.describe_launch("mtx", bits, 1, M, K, S, g)
+    assert "tile=256x128,plain> tiles=160 ksplit=3" in tiles, tiles
+    kw = {} if bits == 4 else dict(scale_range=(0.004, 0.08), zero_const=3.5)
+    p = O.make_problem(K=K, S=S, M=1, bits=bits, group_size=g, seed=3, **kw)
+    xs = np.random.default_rng(6).standard_normal((1, M, K), dtype=np.float32).astype(np.float16)
+    pm = dict(p, M=M, states=xs)
+    d = H.dev_problem(pm)
+    out = H.run_capi(pm, d, "mtx", outs_init=np.full((1, M, S), 5.0, np.float16))
+    _matmul_rows_against_oracle(H, pm, out, np.array([0, 1, 127, 128, 255, 256, 511, 512, 767, 1023, 1024, 1150, 1151]))
+    H.capi.tune(6, 1)
+    try:
+        ref = H.run_capi(pm, d, "mtx")
+    finally:
+        H.capi.tune(6, 0)
+    assert O.max_rel_error(ref.astype(np.float64), out) < H.TOL_EXACT_MTX
