@@ -964,20 +964,25 @@ static WidePlan plan_wide(int64_t R, int64_t K, int64_t S, bool sparse, int64_t 
         return p;
     // measured against the kernel above (K = 2048 ... 20480, S = 1024 ... 28672): with 17 ... 32 rows it
     // needs 32 ... 96 strips and long shares of K, with 33 ... 64 rows matrices of 32 M weights and more
-    // and from 129 rows on the tile kernels win on wide outputs
+    // and from 129 rows on the tile kernels win on wide outputs (beyond 14336 columns; from 193 rows beyond
+    // 10240, from 257 rows beyond 8192 -- K=8192, S=10240, 192 rows: 52 against 64 us; K=4096, S=14336, 192
+    // rows: 42.5 against 49, 256 rows: 52 against 50)
     // (16:32, whose decode costs more here and in the tile kernels alike: 17 ... 32 rows from 64 M weights
-    // on, 33 ... 64 rows from 32 M, 65 ... 128 rows always, beyond that for narrow outputs)
+    // on, 33 ... 64 rows from 32 M, 65 ... 128 rows always, up to 256 rows for outputs of at most 8192 columns
+    // -- K=S=8192, 192 rows: 59 against 71 us --, beyond that of at most 4096)
     if (knob < 2 && forced < 1) {
         if (sparse) {
             if (R <= 32 && K * S < (1ll << 26)) return p;
             if (R > 32 && R <= 64 && K * S < (1ll << 25)) return p;
             // (the padded 256-row tiles win on very wide outputs against two row blocks)
             if (R > 96 && R <= 128 && S > 16384 && p.row_blocks > 1) return p;
-            if (R > 128 && (S > 5120 || (R > 192 && S > 4096))) return p;
+            if (R > 128 && (S > 8192 || (R > 256 && S > 4096))) return p;
         } else {
             if (R <= 32 && (wgs < 32 || wgs > 96 || p.units_per_split < 16)) return p;
             if (R > 32 && R <= 64 && K * S < (1ll << 25)) return p;
-            if (R > 128 && S > 8192) return p;
+            // (beyond 8192 columns only in row blocks of 96 / 128 rows: K=2048, S=12288, 192 rows in three blocks of
+            // 64: 37 against 32 us)
+            if (R > 128 && S > 8192 && (S > (R <= 192 ? 14336 : R <= 256 ? 10240 : 8192) || p.block_rows <= 64)) return p;
         }
     }
     p.part_bytes = p.ksplit > 1 ? (size_t)wgs * 8 * p.ksplit * (2 * p.mt * 4 * 256) : 0;

@@ -74,6 +74,12 @@ def test_few_rows_and_batches():
     assert d("mtx", 4, 1, 96, K, S, 64, sparse=True).startswith("wide_rows_kernel<bits=4,16:32,row_tiles=6> strips=80 row_blocks=1 ksplit=3")
     assert d("mtx", 4, 1, 128, K, S, 64, sparse=True).startswith("wide_rows_kernel<bits=4,16:32,row_tiles=8> strips=80 row_blocks=1 ksplit=3")
     assert d("mtx", 4, 1, 128, 8192, 8192, 64, sparse=True).startswith("wide_rows_kernel<bits=4,16:32,row_tiles=4> strips=32 row_blocks=2 ksplit=4")
+    # 129 ... 256 rows: also on wider outputs (up to 14336 / 10240 columns) in row blocks of 96 / 128 rows
+    assert d("mtx", 4, 1, 192, 4096, 14336, 128).startswith("wide_rows_kernel<bits=4,dense,row_tiles=6> strips=56 row_blocks=2 ksplit=2")
+    assert d("mtx", 4, 1, 256, 4096, 14336, 128).startswith("matmul_kernel_pipe<bits=4,dense,tile=256x128")
+    assert d("mtx", 4, 1, 192, 2048, 12288, 128).startswith("matmul_kernel_pipe<bits=4,dense,tile=256x128")
+    assert d("mtx", 4, 1, 192, K, S, 128).startswith("matmul_kernel_pipe<bits=4,dense,tile=256x128")
+    assert d("mtx", 4, 1, 192, 8192, 8192, 64, sparse=True).startswith("wide_rows_kernel<bits=4,16:32,row_tiles=6> strips=32 row_blocks=2 ksplit=4")
     # up to 512 rows on outputs of at most 8192 columns; wider outputs and the 16:32 format go to the tile kernels
     assert d("mtx", 4, 1, 384, 4096, 4096, 128).startswith("wide_rows_kernel<bits=4,dense,row_tiles=4> strips=16 row_blocks=6 ksplit=2")
     assert d("mtx", 4, 1, 384, K, S, 128).startswith("matmul_kernel_pipe<bits=4,dense,tile=128x256")
