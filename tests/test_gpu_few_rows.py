@@ -415,3 +415,15 @@ def test_tall_row_blocks_sparse_full_size_split_k(H):
     assert "wide_rows_kernel<bits=4,16:32,row_tiles=8> strips=80 row_blocks=1 ksplit=3" in tiles, tiles
     p = O.make_problem(bits=4, K=5120, S=20480, M=128, group_size=64, sparse=True, seed=9)
     _check(H, p, "mtx")
+
+
+@pytest.mark.parametrize("bits,sparse", [(4, False), (3, False), (4, True)])
+def test_many_batch_elements_through_the_matvec_entry(H, bits, sparse):
+    """300 batch elements of one row each: the matvec entry flattens them into rows of the shared-staging kernel
+    and adds onto the prior contents of outs"""
+    g = 64 if sparse else 128
+    assert "wide_rows_kernel" in H.capi.describe_launch("vec", bits, 300, 1, 1024, 512, g, sparse=sparse)
+    kw = {} if bits == 4 else dict(scale_range=(0.004, 0.08), zero_const=3.5)
+    p = O.make_problem(bits=bits, K=1024, S=512, M=1, B=300, group_size=g, sparse=sparse, seed=77, **kw)
+    prior = np.random.default_rng(8).standard_normal((300, 1, 512)).astype(np.float16)
+    _check(H, p, "vec", prior=prior)
