@@ -1099,9 +1099,12 @@ static SkinnySplit plan_skinny_split(int64_t R, int64_t K, int64_t S, bool spars
 
 size_t skinny_workspace_bytes(int64_t R, int64_t K, int64_t S, bool sparse) {
     const SkinnySplit p = plan_skinny_split(R, K, S, sparse);
-    // (the split of the wide kernel can depend on the group size: room for the smallest groups and for one)
-    const WidePlan w1 = plan_wide(R, K, S, sparse, 1), wn = plan_wide(R, K, S, sparse, 0x7FFFFFF);
-    const size_t wide = std::max<size_t>(w1.use ? w1.part_bytes : 0, wn.use ? wn.part_bytes : 0);
+    // (the split of the wide kernel can depend on the group size: room for whichever needs most)
+    size_t wide = 0;
+    for (const int64_t group_units : {1, 2, 3, 4, 6, 8, 16, 0x7FFFFFF}) {
+        const WidePlan w = plan_wide(R, K, S, sparse, group_units);
+        if (w.use) wide = std::max(wide, w.part_bytes);
+    }
     return std::max<size_t>(p.ksplit > 1 ? p.part_bytes : 0, wide);
 }
 
