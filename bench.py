@@ -207,9 +207,9 @@ def main():
                                        "traffic": MATMUL_TRAFFIC_BYTES},
                           "max_rel_err_vs_fp32_oracle": float(f"{mm_err:.3e}")}
 
-        # ---- the few-row products in between (a batch of decoding requests): 8 and 64 rows, same weights
+        # ---- the few-row products in between (a batch of decoding requests): 2, 8 and 64 rows, same weights
         few = {}
-        for rows in (8, 64):
+        for rows in (2, 8, 64):
             xr = xs[:, :rows].contiguous()
             orow = torch.zeros((1, rows, S), dtype=torch.float16, device=dev)
             ws_r = capi.new_matmul_workspace(1, rows, K, S)
@@ -221,7 +221,7 @@ def main():
             few[f"rows_{rows}"] = {"us": round(us, 2), "GB/s": round(nb / (us * 1e-6) / 1e9, 1),
                                    "frac_of_hbm_peak": round(nb / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
                                    "max_rel_err_vs_fp32_oracle": float(f"{err_r:.3e}")}
-        result["few_rows"] = {"workload": "int4 dense, K(N)=5120 S=20480 group=128, 8 and 64 rows of states "
+        result["few_rows"] = {"workload": "int4 dense, K(N)=5120 S=20480 group=128, 2, 8 and 64 rows of states "
                                           "(weights warm in the last-level cache)", **few}
 
     # ---- CPU baseline: torch dequantise + fp32 matmul on the host (reported only)

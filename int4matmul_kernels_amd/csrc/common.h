@@ -118,6 +118,10 @@ bool is_noting();
 bool skinny_rows(int bits, _Float16* outs, const uint32_t* matrix, const _Float16* x, const _Float16* scales,
                  const _Float16* zeros, int64_t R, int64_t K, int64_t S, int64_t group_size, bool accumulate,
                  hipStream_t st, const uint32_t* sparse_mask, void* workspace, size_t workspace_bytes);
+// two to four rows through the matvec kernel (dense formats; csrc/matvec.hip): false when it does not take the shape
+bool matvec_rows(int bits, _Float16* outs, const uint32_t* matrix, const _Float16* x, const _Float16* scales,
+                 const _Float16* zeros, int64_t R, int64_t K, int64_t S, int64_t group_size, bool accumulate,
+                 hipStream_t st, void* workspace, size_t workspace_bytes);
 // most rows the few-row path takes (beyond 96: only its kernel with shared staging, for the shapes it serves)
 constexpr int SK_WIDE_MAX_ROWS = 512;
 // bytes of partial tiles with which the few-row kernel splits K across workgroups (0: no split)

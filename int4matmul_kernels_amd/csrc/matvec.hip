@@ -31,6 +31,7 @@
 // slots.  No cache-wide fence and no read-modify-write atomics are used.
 #include "common.h"
 
+#include <algorithm>
 #include <mutex>
 
 namespace i4 {
@@ -55,6 +56,8 @@ struct MatvecArgs {
     uint32_t* sticky;       // hand-over error word of the workspace (non-zero: poisoned)
     int spin_limit;         // polls before a reader gives up
     uint64_t* timeline;     // instrumented variant only: 16 time stamps per wave (8 wave slots per workgroup)
+    int rows;               // several rows of states in one pass (NR = 4 kernels): how many (2 .. 4), K apart in x, S apart in outs
+    int accumulate;         // ... and whether they add onto outs (the matvec entry) or overwrite it (the matmul entry)
 };
 
 // ------------------------------------------------------------------ formats
@@ -399,10 +402,19 @@ __device__ __forceinline__ uint64_t slot_load(const uint64_t* p) {
 // entry (0), after its first requests (1), after the staging barrier (2), after each of its first
 // nine units (3..11), after the workgroup's reduction (12) and at the end (13), and the hardware
 // ids of where it ran (15).
-template <int BITS, bool SPARSE, int LK, bool PF, bool TL = false>
+//
+// NR = 4: up to four rows of states in one pass over the weights (dense formats).  The 4x4x4 MFMA
+// computes a 4 x 4 block per four lanes; with one row of states every lane passes the same four
+// states as its row of A and three of the four result registers repeat the first.  Here lane
+// 4b + i passes row i's states, and register i of a lane is row i's dot product for the lane's
+// column: the same instructions and the same weight traffic give four rows of outputs.  Staged
+// states, unit sums, the reduction area and the hand-over slots (slot row = split * 4 + row) are
+// kept per row.
+template <int BITS, bool SPARSE, int LK, bool PF, bool TL = false, int NR = 1>
 __global__ __launch_bounds__(MV_MAX_WAVES * WAVE)
 void matvec_kernel(MatvecArgs a) {
     constexpr bool FAST = Fmt<BITS, SPARSE>::FAST;
+    static_assert(NR == 1 || (NR == 4 && FAST && !SPARSE && !TL), "four rows: dense formats only");
     constexpr int LC = WAVE / LK;                 // column lanes per lane group
     constexpr int COLS = LC * 4;                  // columns per strip
 
@@ -413,7 +425,7 @@ void matvec_kernel(MatvecArgs a) {
     // its LDS address is a compile-time constant (a table read then needs no address add)
     __shared__ __attribute__((aligned(16))) u32x4 lut[SPARSE ? 256 : 1];
     h16* xs = reinterpret_cast<h16*>(smem);
-    float* sums = reinterpret_cast<float*>(smem + (size_t)a.units_per_wg * Fmt<BITS, SPARSE>::XS);
+    float* sums = reinterpret_cast<float*>(smem + (size_t)a.units_per_wg * NR * Fmt<BITS, SPARSE>::XS);
     float* red = reinterpret_cast<float*>(smem);
 
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6, nwaves = blockDim.x >> 6;
@@ -445,7 +457,9 @@ void matvec_kernel(MatvecArgs a) {
     constexpr int ITEM_H = SPARSE ? 32 : (BITS == 4 ? 8 : (BITS == 2 ? 16 : 32));   // halves per item
     constexpr int IPU = 64 / ITEM_H;                                  // items per unit
     constexpr int ITEM_V = ITEM_H / 8;                                // 16-byte loads per item
-    const int nitems = FAST ? (wg_u1 - wg_u0) * IPU : 0;
+    // (NR rows: item r belongs to unit-row block r / IPU = unit * NR + row, whose staged states and sums
+    // lie side by side; rows beyond a.rows are staged as zeros)
+    const int nitems = FAST ? (wg_u1 - wg_u0) * IPU * NR : 0;
     const int nitems8 = (nitems + 7) & ~7;
     const h16* xg = a.x + wg_u0 * 64;
     u32x4 xv[ITEM_V];
@@ -453,8 +467,16 @@ void matvec_kernel(MatvecArgs a) {
     for (int i = 0; i < ITEM_V; ++i) xv[i] = u32x4{0, 0, 0, 0};
     auto load_x = [&](int r) {
         if (r < nitems) {
+            if constexpr (NR == 1) {
 #pragma unroll
-            for (int i = 0; i < ITEM_V; ++i) xv[i] = *reinterpret_cast<const u32x4*>(xg + r * ITEM_H + i * 8);
+                for (int i = 0; i < ITEM_V; ++i) xv[i] = *reinterpret_cast<const u32x4*>(xg + r * ITEM_H + i * 8);
+            } else {
+                const int block = r / IPU, row = block % NR, item = (block / NR) * IPU + r % IPU;
+#pragma unroll
+                for (int i = 0; i < ITEM_V; ++i)
+                    xv[i] = row < a.rows ? *reinterpret_cast<const u32x4*>(xg + (int64_t)row * a.K + item * ITEM_H + i * 8)
+                                         : u32x4{0, 0, 0, 0};
+            }
         }
     };
     if constexpr (FAST) load_x(t);
@@ -575,6 +597,7 @@ void matvec_kernel(MatvecArgs a) {
     stamp(2);
 
     float y[4] = {0.f, 0.f, 0.f, 0.f};
+    float yr[NR == 1 ? 1 : 4][NR == 1 ? 1 : NR] = {};       // NR rows: yr[column][row] instead of y
     bool need_general = false;
 
     auto finish_unit = [&](const Unit<BITS, SPARSE>& un, int unit) {
@@ -599,14 +622,28 @@ void matvec_kernel(MatvecArgs a) {
 #pragma unroll
             for (int c = 0; c < 4; ++c) acc[c] = f32x4{0.f, 0.f, 0.f, 0.f};
             const int lu = unit - wg_u0;
-            unit_fast(un, xs + lu * (Fmt<BITS, SPARSE>::XS / 2), acc);
-            const float xsum = sums[lu * 2], xoff = sums[lu * 2 + 1];
+            if constexpr (NR == 1) {
+                unit_fast(un, xs + lu * (Fmt<BITS, SPARSE>::XS / 2), acc);
+                const float xsum = sums[lu * 2], xoff = sums[lu * 2 + 1];
 #pragma unroll
-            for (int c = 0; c < 4; ++c) {
-                // exponent-mode columns (scale < 0 or NaN) contribute nothing here
-                const float sl = fmaxf(sc[c], 0.f);
-                y[c] += sl * ((acc[c][0] - xoff) - ze[c] * xsum);
-                need_general |= expo[c];
+                for (int c = 0; c < 4; ++c) {
+                    // exponent-mode columns (scale < 0 or NaN) contribute nothing here
+                    const float sl = fmaxf(sc[c], 0.f);
+                    y[c] += sl * ((acc[c][0] - xoff) - ze[c] * xsum);
+                    need_general |= expo[c];
+                }
+            } else {
+                unit_fast(un, xs + (lu * NR + (lane & 3)) * (Fmt<BITS, SPARSE>::XS / 2), acc);
+                float xsum[NR], xoff[NR];
+#pragma unroll
+                for (int r = 0; r < NR; ++r) { xsum[r] = sums[(lu * NR + r) * 2]; xoff[r] = sums[(lu * NR + r) * 2 + 1]; }
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    const float sl = fmaxf(sc[c], 0.f);
+#pragma unroll
+                    for (int r = 0; r < NR; ++r) yr[c][r] += sl * ((acc[c][r] - xoff[r]) - ze[c] * xsum[r]);
+                    need_general |= expo[c];
+                }
             }
         } else {
             float acc[4], xsv[4];
@@ -669,10 +706,20 @@ void matvec_kernel(MatvecArgs a) {
 #pragma unroll
                     for (int c = 0; c < 4; ++c) acc[c] = f32x4{0.f, 0.f, 0.f, 0.f};
                     const int lu = v - wg_u0;
-                    unit_fast<true>(ua, xs + lu * (Fmt<BITS, SPARSE>::XS / 2), acc);
-                    const float xsum = sums[lu * 2];
+                    if constexpr (NR == 1) {
+                        unit_fast<true>(ua, xs + lu * (Fmt<BITS, SPARSE>::XS / 2), acc);
+                        const float xsum = sums[lu * 2];
 #pragma unroll
-                    for (int c = 0; c < 4; ++c) y[c] += expo[c] ? ze[c] * xsum - sc[c] * acc[c][0] : 0.f;
+                        for (int c = 0; c < 4; ++c) y[c] += expo[c] ? ze[c] * xsum - sc[c] * acc[c][0] : 0.f;
+                    } else {
+                        unit_fast<true>(ua, xs + (lu * NR + (lane & 3)) * (Fmt<BITS, SPARSE>::XS / 2), acc);
+#pragma unroll
+                        for (int r = 0; r < NR; ++r) {
+                            const float xsum = sums[(lu * NR + r) * 2];
+#pragma unroll
+                            for (int c = 0; c < 4; ++c) yr[c][r] += expo[c] ? ze[c] * xsum - sc[c] * acc[c][r] : 0.f;
+                        }
+                    }
                 } else {
                     if (!(expo[0] | expo[1] | expo[2] | expo[3])) continue;
                     float acc[4], xsv[4];
@@ -682,6 +729,58 @@ void matvec_kernel(MatvecArgs a) {
                 }
             }
         }
+    }
+
+    if constexpr (NR > 1) {
+        // ---- the same reduction and hand-over per row: a plane of the reduction area and a slot row per row
+        __syncthreads();
+        const int plane = (int)blockDim.x * 4;
+#pragma unroll
+        for (int r = 0; r < NR; ++r)
+            *reinterpret_cast<f32x4*>(&red[r * plane + (wave * 64 + lane) * 4]) = f32x4{yr[0][r], yr[1][r], yr[2][r], yr[3][r]};
+        __syncthreads();
+        constexpr int MAXC = COLS / WAVE;
+        const uint32_t poisoned = a.splits > 1 && split == a.splits - 1
+                                      ? __hip_atomic_load(a.sticky, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0u;
+        for (int r = 0; r < a.rows; ++r) {
+#pragma unroll
+            for (int i = 0; i < MAXC; ++i) {
+                const int j = t + i * (int)blockDim.x;
+                const int ocol = strip * COLS + j;
+                if (j >= COLS || ocol >= a.S) continue;
+                float total = 0.f;
+                for (int w = 0; w < nwaves; ++w)
+#pragma unroll
+                    for (int k = 0; k < LK; ++k) total += red[r * plane + (w * 64 + k * LC) * 4 + j];
+                h16* const out = a.outs + (int64_t)r * a.S + ocol;
+                const float prior = a.accumulate ? (float)*out : 0.f;
+                if (a.splits == 1) {
+                    *out = (h16)(prior + total);
+                } else if (split != a.splits - 1) {
+                    slot_store(&a.slots[((int64_t)split * NR + r) * a.S + ocol], total, SLOT_FULL);
+                } else {
+                    float sum = prior;
+                    bool ok = poisoned == 0;
+                    for (int sp = 0; sp < a.splits - 1; ++sp) {
+                        uint64_t* p = &a.slots[((int64_t)sp * NR + r) * a.S + ocol];
+                        uint64_t v = slot_load(p);
+                        int spins = 0;
+                        while ((uint32_t)(v >> 32) != SLOT_FULL && spins < a.spin_limit) {
+                            __builtin_amdgcn_s_sleep(1);
+                            v = slot_load(p);
+                            ++spins;
+                        }
+                        ok &= (uint32_t)(v >> 32) == SLOT_FULL;
+                        sum += bitcast<float>((uint32_t)v);
+                        slot_store(p, 0.f, 0u);
+                    }
+                    sum += total;
+                    if (!ok) __hip_atomic_store(a.sticky, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    *out = ok ? (h16)sum : (h16)__builtin_nanf("");
+                }
+            }
+        }
+        return;
     }
 
     // ---- workgroup reduction through LDS (the staging area is free now)
@@ -765,10 +864,26 @@ void matvec_kernel(MatvecArgs a) {
     stamp(13); stamp(15);
 }
 
+// LDS of a launch: staged states + per-unit sums (per row), or the reduction area (4 floats per thread and row)
+template <int BITS, bool SPARSE>
+static size_t matvec_lds_bytes(int units_per_wg, int threads, int nr) {
+    return std::max((size_t)units_per_wg * nr * (Fmt<BITS, SPARSE>::XS + 8), (size_t)threads * 16 * nr);
+}
+
+// up to four rows of states per pass (dense formats, no prefetch variant needed: the launcher passes its choice)
+template <int BITS>
+static void launch_rows(const MatvecArgs& a, int lk, bool pf, dim3 grid, dim3 block, hipStream_t st) {
+    const size_t lds = matvec_lds_bytes<BITS, false>(a.units_per_wg, (int)block.x, 4);
+#define I4_LAUNCH(LK_, PF_) hipLaunchKernelGGL((matvec_kernel<BITS, false, LK_, PF_, false, 4>), grid, block, lds, st, a)
+    if (lk == 1) { if (pf) I4_LAUNCH(1, true); else I4_LAUNCH(1, false); }
+    else if (lk == 2) { if (pf) I4_LAUNCH(2, true); else I4_LAUNCH(2, false); }
+    else { if (pf) I4_LAUNCH(4, true); else I4_LAUNCH(4, false); }
+#undef I4_LAUNCH
+}
+
 template <int BITS, bool SPARSE>
 static void launch(const MatvecArgs& a, int lk, bool pf, dim3 grid, dim3 block, hipStream_t st) {
-    size_t lds = (size_t)a.units_per_wg * (Fmt<BITS, SPARSE>::XS + 8);     // staged states + per-unit sums
-    if (lds < (size_t)block.x * 16) lds = (size_t)block.x * 16;           // reduction area: 4 floats per thread
+    const size_t lds = matvec_lds_bytes<BITS, SPARSE>(a.units_per_wg, (int)block.x, 1);
 #define I4_LAUNCH(LK_, PF_) do { \
         if constexpr (BITS == 4 && !SPARSE) { \
             if (a.timeline) { hipLaunchKernelGGL((matvec_kernel<BITS, SPARSE, LK_, PF_, true>), grid, block, lds, st, a); break; } \
@@ -785,24 +900,10 @@ static void launch(const MatvecArgs& a, int lk, bool pf, dim3 grid, dim3 block, 
 
 using namespace i4;
 
-static int matvec_impl(int bits, void* outs, const void* matrix, const void* multiplier,
-                       const void* scales, const void* zeros, const void* sparse_mask,
-                       const int4mm_shape* shape, void* workspace, size_t workspace_bytes,
-                       void* stream) {
-    int rc = validate_product(bits, outs, matrix, multiplier, scales, zeros, sparse_mask, shape, true);
-    if (rc != INT4MM_OK) return rc;
-    const int64_t B = shape->batch, K = shape->in_size, S = shape->out_size;
-    if (B * shape->seq_len * S == 0) return INT4MM_OK;
-
-    const int units_total = (int)(K / 64);
-    const int64_t g = shape->group_size < 0 ? ONE_GROUP : shape->group_size;
-
-    // several batch elements of one row each: one pass over the weights for all of them
-    if (B >= 2 && B <= SK_WIDE_MAX_ROWS && !tuning(TUNE_NO_SKINNY) &&
-        skinny_rows(bits, (h16*)outs, (const uint32_t*)matrix, (const h16*)multiplier, (const h16*)scales,
-                    (const h16*)zeros, B, K, S, g, true, (hipStream_t)stream, (const uint32_t*)sparse_mask, workspace, workspace_bytes))
-        return check_launch("matvec");
-
+// Launch shape of a matvec: strips of 256 / lk columns, `waves` waves per workgroup, `upwg` units per
+// workgroup dealt round-robin to its lane groups; the grid's y dimension (`splits`) covers the rest of K.
+struct MatvecShape { int lk, waves, upwg, splits, strips; };
+static MatvecShape plan_matvec(int64_t S, int units_total) {
     // Launch shape: strips of 256/lk columns, `waves` waves per workgroup, `upwg`
     // units per workgroup dealt round-robin to its lane groups; the grid's y
     // dimension covers the rest of K.
@@ -853,6 +954,81 @@ static int matvec_impl(int bits, void* outs, const void* matrix, const void* mul
         splits = (units_total + upwg - 1) / upwg;
     }
     if (waves * lk > upwg) waves = (upwg + lk - 1) / lk;    // no idle waves
+    return MatvecShape{lk, waves, upwg, splits, strips};
+}
+
+// Two to four rows of states (a matmul with that many rows in all, or a matvec with that many batch
+// elements), dense formats: the matvec kernel with a row per MFMA result register -- one pass over the
+// weights at the matvec's rate.  Returns false when it does not take the shape (the few-row kernels do then):
+// the hand-over needs four slot rows per split, the staged states four times the LDS.
+bool i4::matvec_rows(int bits, h16* outs, const uint32_t* matrix, const h16* x, const h16* scales, const h16* zeros,
+                     int64_t R, int64_t K, int64_t S, int64_t group_size, bool accumulate, hipStream_t st,
+                     void* workspace, size_t workspace_bytes) {
+    if (R < 2 || R > 4 || K % 64 != 0 || S % 4 != 0 || tuning(TUNE_MV_TIMELINE)) return false;
+    // measured against the few-row kernel (S = 11008 ... 32768, warm weights): 10 - 26 % faster up to K = 5120
+    // (K=5120, S=20480: 2 / 3 / 4 rows 14.0 / 15.4 / 17.1 against 18.4 / 18.1 / 18.3 us; K=4096, S=11008: 9.5 / 11.1 /
+    // 12.3 against 11.3 / 12.5 / 12.4), 3 - 14 % slower from K = 6144 on, where staging four rows of states per
+    // workgroup weighs more; below K = 4096 only two rows gain
+    if (K > 5120 || (R > 2 && K < 4096)) return false;
+    const int units_total = (int)(K / 64);
+    const MatvecShape ms = plan_matvec(S, units_total);
+    if (ms.splits * 4 > MV_MAX_SPLITS || ms.upwg * 4 > MV_MAX_UNITS_WG) return false;
+    const WorkspaceParts ws = workspace_parts(workspace, workspace_bytes);
+    if (ms.splits > 1 && ws.slots_bytes < matvec_slots_bytes(S)) return false;
+    const bool pf = ms.upwg >= 3 * ms.waves * ms.lk && tuning(TUNE_MV_NOPF) == 0;
+    MatvecArgs a;
+    a.outs = outs;
+    a.matrix = matrix;
+    a.mask = nullptr;
+    a.x = x;
+    a.scales = scales;
+    a.zeros = zeros;
+    a.slots = (uint64_t*)workspace;
+    a.K = (int)K;
+    a.S = (int)S;
+    a.units_total = units_total;
+    a.units_per_wg = ms.upwg;
+    a.group_units = (int)(group_size / 64 > 0x7FFFFFF ? 0x7FFFFFF : group_size / 64);
+    a.splits = ms.splits;
+    a.timeline = nullptr;
+    a.sticky = ms.splits > 1 ? reinterpret_cast<uint32_t*>(ws.counters - 8) : nullptr;
+    a.spin_limit = tuning(TUNE_MV_SPIN) > 0 ? (int)tuning(TUNE_MV_SPIN) : MV_SPIN_LIMIT;
+    a.rows = (int)R;
+    a.accumulate = accumulate ? 1 : 0;
+    const dim3 grid(ms.strips, ms.splits, 1), block(ms.waves * WAVE);
+    if (noting("matvec_kernel<bits=%d,dense,lane_groups=%d,prefetch=%d,rows=4> strips=%d splits=%d waves=%d units_per_workgroup=%d rows=%d",
+               bits, ms.lk, (int)pf, ms.strips, ms.splits, ms.waves, ms.upwg, (int)R))
+        return true;
+    if (bits == 4) launch_rows<4>(a, ms.lk, pf, grid, block, st);
+    else if (bits == 3) launch_rows<3>(a, ms.lk, pf, grid, block, st);
+    else launch_rows<2>(a, ms.lk, pf, grid, block, st);
+    return true;
+}
+
+static int matvec_impl(int bits, void* outs, const void* matrix, const void* multiplier,
+                       const void* scales, const void* zeros, const void* sparse_mask,
+                       const int4mm_shape* shape, void* workspace, size_t workspace_bytes,
+                       void* stream) {
+    int rc = validate_product(bits, outs, matrix, multiplier, scales, zeros, sparse_mask, shape, true);
+    if (rc != INT4MM_OK) return rc;
+    const int64_t B = shape->batch, K = shape->in_size, S = shape->out_size;
+    if (B * shape->seq_len * S == 0) return INT4MM_OK;
+
+    const int units_total = (int)(K / 64);
+    const int64_t g = shape->group_size < 0 ? ONE_GROUP : shape->group_size;
+
+    // several batch elements of one row each: one pass over the weights for all of them
+    if (B >= 2 && B <= 4 && !sparse_mask && !tuning(TUNE_NO_SKINNY) &&
+        matvec_rows(bits, (h16*)outs, (const uint32_t*)matrix, (const h16*)multiplier, (const h16*)scales, (const h16*)zeros,
+                    B, K, S, g, true, (hipStream_t)stream, workspace, workspace_bytes))
+        return check_launch("matvec");
+    if (B >= 2 && B <= SK_WIDE_MAX_ROWS && !tuning(TUNE_NO_SKINNY) &&
+        skinny_rows(bits, (h16*)outs, (const uint32_t*)matrix, (const h16*)multiplier, (const h16*)scales,
+                    (const h16*)zeros, B, K, S, g, true, (hipStream_t)stream, (const uint32_t*)sparse_mask, workspace, workspace_bytes))
+        return check_launch("matvec");
+
+    const MatvecShape ms = plan_matvec(S, units_total);
+    const int lk = ms.lk, waves = ms.waves, upwg = ms.upwg, splits = ms.splits, strips = ms.strips;
     if (upwg > MV_MAX_UNITS_WG) return INT4MM_ERR_SHAPE;
     if (splits > 1 && workspace_parts(workspace, workspace_bytes).slots_bytes < matvec_slots_bytes(S))
         return INT4MM_ERR_WORKSPACE;
@@ -874,6 +1050,8 @@ static int matvec_impl(int bits, void* outs, const void* matrix, const void* mul
     a.timeline = (uint64_t*)(uintptr_t)tuning(TUNE_MV_TIMELINE);
     a.sticky = splits > 1 ? reinterpret_cast<uint32_t*>(workspace_parts(workspace, workspace_bytes).counters - 8) : nullptr;
     a.spin_limit = tuning(TUNE_MV_SPIN) > 0 ? (int)tuning(TUNE_MV_SPIN) : MV_SPIN_LIMIT;
+    a.rows = 1;
+    a.accumulate = 1;
 
     const dim3 grid(strips, splits, 1), block(waves * WAVE);
     hipStream_t st = (hipStream_t)stream;

@@ -60,6 +60,19 @@ def test_long_k_on_a_narrow_output():
     assert "tile=128x256" in d("mtx", 4, 1, 1024, S, K, 128, workspace_bytes=0)
 
 
+def test_two_to_four_rows_take_the_matvec_kernel_up_to_k_5120():
+    assert d("mtx", 4, 1, 3, K, S, 128).startswith(
+        "matvec_kernel<bits=4,dense,lane_groups=2,prefetch=0,rows=4> strips=160 splits=4 waves=4 units_per_workgroup=23 rows=3")
+    assert d("vec", 3, 2, 1, K, S, 128).startswith("matvec_kernel<bits=3,dense,lane_groups=2,prefetch=0,rows=4>")
+    assert d("mtx", 4, 2, 2, 4096, 11008, 128).startswith("matvec_kernel<bits=4,dense,lane_groups=4,prefetch=0,rows=4> strips=172 splits=4")
+    assert d("mtx", 4, 1, 3, 8192, 22016, 128).startswith("skinny_kernel")          # long K: the few-row kernel
+    assert d("mtx", 4, 1, 3, 2048, 32768, 128).startswith("skinny_kernel")          # short K: only two rows
+    assert d("mtx", 4, 1, 2, 2048, 32768, 128).startswith("matvec_kernel")
+    assert d("mtx", 4, 1, 5, K, S, 128).startswith("skinny_kernel")
+    assert d("mtx", 4, 1, 3, K, S, 64, sparse=True).startswith("skinny_kernel<bits=4,16:32")
+    assert d("mtx", 4, 1, 3, K, S, 128, workspace_bytes=0).startswith("skinny_kernel")  # no room for the hand-over
+
+
 def test_few_rows_and_batches():
     assert d("mtx", 4, 1, 8, K, S, 128).startswith("skinny_kernel<bits=4,dense,columns_per_lane=4,row_tiles=1> strips=320")
     assert d("vec", 4, 8, 1, K, S, 128).startswith("skinny_kernel<bits=4,dense,columns_per_lane=4,row_tiles=1> strips=320")

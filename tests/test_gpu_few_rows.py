@@ -427,3 +427,49 @@ def test_many_batch_elements_through_the_matvec_entry(H, bits, sparse):
     p = O.make_problem(bits=bits, K=1024, S=512, M=1, B=300, group_size=g, sparse=sparse, seed=77, **kw)
     prior = np.random.default_rng(8).standard_normal((300, 1, 512)).astype(np.float16)
     _check(H, p, "vec", prior=prior)
+
+
+# ---- two to four rows through the matvec kernel (a row of states per MFMA result register; dense formats, K <= 5120)
+@pytest.mark.parametrize("bits", [4, 3, 2])
+@pytest.mark.parametrize("R", [2, 3, 4])
+@pytest.mark.parametrize("K,S,g", [(4096, 5120, 128), (5120, 8192, 64), (4096, 6144, -1)])
+def test_two_to_four_rows_equal_the_matvec_row_by_row(H, bits, R, K, S, g):
+    """the matmul entry (overwrites outs) and the matvec entry with R batch elements (adds onto outs) give, bit for
+    bit, what R calls of the one-row matvec give; exponent-mode columns included"""
+    capi = H.capi
+    assert "rows=4>" in capi.describe_launch("mtx", bits, 1, R, K, S, g)
+    assert "rows=4>" in capi.describe_launch("vec", bits, R, 1, K, S, g)
+    p = _problem(bits, K=K, S=S, M=R, group_size=g, seed=R + K + S)
+    sc = p["scales"].reshape(-1, S)
+    sc[0, 8:12] *= np.float16(-1)
+    sc[-1, S - 1] *= np.float16(-1)
+    d = H.dev_problem(p)
+    exact, f32 = H.oracles(p)
+    got = H.run_capi(p, d, "mtx", outs_init=np.full((1, R, S), 7.0, np.float16))
+    H.assert_product_close(got, exact, f32, kind="vec")
+    ws = capi.new_matmul_workspace(1, R, K, S, False)
+    rows = torch.zeros((1, R, S), dtype=torch.float16, device="cuda")
+    for r in range(R):
+        capi.matvec(bits, rows[:, r:r + 1], d["matrix"], d["states"][:, r:r + 1].contiguous(), d["scales"], d["zeros"], g, None, ws)
+    torch.cuda.synchronize()
+    assert np.array_equal(got, rows.cpu().numpy())
+    # the matvec entry: R batch elements, prior contents of outs added
+    prior = np.random.default_rng(R).standard_normal((R, 1, S)).astype(np.float16)
+    outs = torch.from_numpy(prior).cuda()
+    want = torch.from_numpy(prior).cuda()
+    xb = d["states"].reshape(R, 1, K).contiguous()
+    capi.matvec(bits, outs, d["matrix"], xb, d["scales"], d["zeros"], g, None, ws)
+    for r in range(R):
+        capi.matvec(bits, want[r:r + 1], d["matrix"], xb[r:r + 1], d["scales"], d["zeros"], g, None, ws)
+    torch.cuda.synchronize()
+    assert np.array_equal(outs.cpu().numpy(), want.cpu().numpy())
+
+
+@pytest.mark.parametrize("bits", [4, 3, 2])
+def test_two_to_four_rows_full_size(H, bits):
+    """K=5120, S=20480, three rows: 160 strips, four splits of K handing over three slot rows each"""
+    assert "rows=4> strips=160 splits=4" in H.capi.describe_launch("mtx", bits, 1, 3, 5120, 20480, 128)
+    p = _problem(bits, K=5120, S=20480, M=3, group_size=128, seed=12)
+    _check(H, p, "mtx")
+    again = _problem(bits, K=5120, S=20480, M=2, group_size=128, seed=13)       # the slots come back clean
+    _check(H, again, "mtx")
