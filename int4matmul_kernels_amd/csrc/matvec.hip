@@ -403,18 +403,18 @@ __device__ __forceinline__ uint64_t slot_load(const uint64_t* p) {
 // nine units (3..11), after the workgroup's reduction (12) and at the end (13), and the hardware
 // ids of where it ran (15).
 //
-// NR = 4: up to four rows of states in one pass over the weights (dense formats).  The 4x4x4 MFMA
+// NR = 2, 4: up to two / four rows of states in one pass over the weights (dense formats).  The 4x4x4 MFMA
 // computes a 4 x 4 block per four lanes; with one row of states every lane passes the same four
 // states as its row of A and three of the four result registers repeat the first.  Here lane
 // 4b + i passes row i's states, and register i of a lane is row i's dot product for the lane's
-// column: the same instructions and the same weight traffic give four rows of outputs.  Staged
-// states, unit sums, the reduction area and the hand-over slots (slot row = split * 4 + row) are
-// kept per row.
+// column: the same instructions and the same weight traffic give four rows of outputs (NR = 2:
+// lanes 4b + i and 4b + i + 2 pass row i, two registers are used).  Staged states, unit sums, the
+// reduction area and the hand-over slots (slot row = split * NR + row) are kept per row.
 template <int BITS, bool SPARSE, int LK, bool PF, bool TL = false, int NR = 1>
 __global__ __launch_bounds__(MV_MAX_WAVES * WAVE)
 void matvec_kernel(MatvecArgs a) {
     constexpr bool FAST = Fmt<BITS, SPARSE>::FAST;
-    static_assert(NR == 1 || (NR == 4 && FAST && !SPARSE && !TL), "four rows: dense formats only");
+    static_assert(NR == 1 || ((NR == 2 || NR == 4) && FAST && !SPARSE && !TL), "several rows: dense formats only");
     constexpr int LC = WAVE / LK;                 // column lanes per lane group
     constexpr int COLS = LC * 4;                  // columns per strip
 
@@ -633,7 +633,7 @@ void matvec_kernel(MatvecArgs a) {
                     need_general |= expo[c];
                 }
             } else {
-                unit_fast(un, xs + (lu * NR + (lane & 3)) * (Fmt<BITS, SPARSE>::XS / 2), acc);
+                unit_fast(un, xs + (lu * NR + (lane & (NR - 1))) * (Fmt<BITS, SPARSE>::XS / 2), acc);
                 float xsum[NR], xoff[NR];
 #pragma unroll
                 for (int r = 0; r < NR; ++r) { xsum[r] = sums[(lu * NR + r) * 2]; xoff[r] = sums[(lu * NR + r) * 2 + 1]; }
@@ -712,7 +712,7 @@ void matvec_kernel(MatvecArgs a) {
 #pragma unroll
                         for (int c = 0; c < 4; ++c) y[c] += expo[c] ? ze[c] * xsum - sc[c] * acc[c][0] : 0.f;
                     } else {
-                        unit_fast<true>(ua, xs + (lu * NR + (lane & 3)) * (Fmt<BITS, SPARSE>::XS / 2), acc);
+                        unit_fast<true>(ua, xs + (lu * NR + (lane & (NR - 1))) * (Fmt<BITS, SPARSE>::XS / 2), acc);
 #pragma unroll
                         for (int r = 0; r < NR; ++r) {
                             const float xsum = sums[(lu * NR + r) * 2];
@@ -871,10 +871,10 @@ static size_t matvec_lds_bytes(int units_per_wg, int threads, int nr) {
 }
 
 // up to four rows of states per pass (dense formats, no prefetch variant needed: the launcher passes its choice)
-template <int BITS>
+template <int BITS, int NR>
 static void launch_rows(const MatvecArgs& a, int lk, bool pf, dim3 grid, dim3 block, hipStream_t st) {
-    const size_t lds = matvec_lds_bytes<BITS, false>(a.units_per_wg, (int)block.x, 4);
-#define I4_LAUNCH(LK_, PF_) hipLaunchKernelGGL((matvec_kernel<BITS, false, LK_, PF_, false, 4>), grid, block, lds, st, a)
+    const size_t lds = matvec_lds_bytes<BITS, false>(a.units_per_wg, (int)block.x, NR);
+#define I4_LAUNCH(LK_, PF_) hipLaunchKernelGGL((matvec_kernel<BITS, false, LK_, PF_, false, NR>), grid, block, lds, st, a)
     if (lk == 1) { if (pf) I4_LAUNCH(1, true); else I4_LAUNCH(1, false); }
     else if (lk == 2) { if (pf) I4_LAUNCH(2, true); else I4_LAUNCH(2, false); }
     else { if (pf) I4_LAUNCH(4, true); else I4_LAUNCH(4, false); }
@@ -968,11 +968,15 @@ bool i4::matvec_rows(int bits, h16* outs, const uint32_t* matrix, const h16* x, 
     // measured against the few-row kernel (S = 11008 ... 32768, warm weights): 10 - 26 % faster up to K = 5120
     // (K=5120, S=20480: 2 / 3 / 4 rows 14.0 / 15.4 / 17.1 against 18.4 / 18.1 / 18.3 us; K=4096, S=11008: 9.5 / 11.1 /
     // 12.3 against 11.3 / 12.5 / 12.4), 3 - 14 % slower from K = 6144 on, where staging four rows of states per
-    // workgroup weighs more; below K = 4096 only two rows gain
-    if (K > 5120 || (R > 2 && K < 4096)) return false;
+    // workgroup weighs more; below K = 4096 only two rows gain.  Two rows (NR = 2) gain on a longer K as well
+    // while K is split at most five ways (K=8192, S=22016: 21.0 against 26.0 us; K=28672, S=8192: 26.6 against
+    // 33.3; ten splits, K=14336, S=4096: 15.5 against 13.3)
+    if (R > 2 && (K > 5120 || K < 4096)) return false;
     const int units_total = (int)(K / 64);
     const MatvecShape ms = plan_matvec(S, units_total);
-    if (ms.splits * 4 > MV_MAX_SPLITS || ms.upwg * 4 > MV_MAX_UNITS_WG) return false;
+    const int nr = R <= 2 ? 2 : 4;
+    if (ms.splits * nr > MV_MAX_SPLITS || ms.upwg * nr > MV_MAX_UNITS_WG) return false;
+    if (R == 2 && K > 5120 && ms.splits > 5) return false;
     const WorkspaceParts ws = workspace_parts(workspace, workspace_bytes);
     if (ms.splits > 1 && ws.slots_bytes < matvec_slots_bytes(S)) return false;
     const bool pf = ms.upwg >= 3 * ms.waves * ms.lk && tuning(TUNE_MV_NOPF) == 0;
@@ -996,12 +1000,18 @@ bool i4::matvec_rows(int bits, h16* outs, const uint32_t* matrix, const h16* x, 
     a.rows = (int)R;
     a.accumulate = accumulate ? 1 : 0;
     const dim3 grid(ms.strips, ms.splits, 1), block(ms.waves * WAVE);
-    if (noting("matvec_kernel<bits=%d,dense,lane_groups=%d,prefetch=%d,rows=4> strips=%d splits=%d waves=%d units_per_workgroup=%d rows=%d",
-               bits, ms.lk, (int)pf, ms.strips, ms.splits, ms.waves, ms.upwg, (int)R))
+    if (noting("matvec_kernel<bits=%d,dense,lane_groups=%d,prefetch=%d,rows=%d> strips=%d splits=%d waves=%d units_per_workgroup=%d rows=%d",
+               bits, ms.lk, (int)pf, nr, ms.strips, ms.splits, ms.waves, ms.upwg, (int)R))
         return true;
-    if (bits == 4) launch_rows<4>(a, ms.lk, pf, grid, block, st);
-    else if (bits == 3) launch_rows<3>(a, ms.lk, pf, grid, block, st);
-    else launch_rows<2>(a, ms.lk, pf, grid, block, st);
+    if (nr == 2) {
+        if (bits == 4) launch_rows<4, 2>(a, ms.lk, pf, grid, block, st);
+        else if (bits == 3) launch_rows<3, 2>(a, ms.lk, pf, grid, block, st);
+        else launch_rows<2, 2>(a, ms.lk, pf, grid, block, st);
+    } else {
+        if (bits == 4) launch_rows<4, 4>(a, ms.lk, pf, grid, block, st);
+        else if (bits == 3) launch_rows<3, 4>(a, ms.lk, pf, grid, block, st);
+        else launch_rows<2, 4>(a, ms.lk, pf, grid, block, st);
+    }
     return true;
 }
 

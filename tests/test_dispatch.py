@@ -63,9 +63,11 @@ def test_long_k_on_a_narrow_output():
 def test_two_to_four_rows_take_the_matvec_kernel_up_to_k_5120():
     assert d("mtx", 4, 1, 3, K, S, 128).startswith(
         "matvec_kernel<bits=4,dense,lane_groups=2,prefetch=0,rows=4> strips=160 splits=4 waves=4 units_per_workgroup=23 rows=3")
-    assert d("vec", 3, 2, 1, K, S, 128).startswith("matvec_kernel<bits=3,dense,lane_groups=2,prefetch=0,rows=4>")
+    assert d("vec", 3, 2, 1, K, S, 128).startswith("matvec_kernel<bits=3,dense,lane_groups=2,prefetch=0,rows=2>")
     assert d("mtx", 4, 2, 2, 4096, 11008, 128).startswith("matvec_kernel<bits=4,dense,lane_groups=4,prefetch=0,rows=4> strips=172 splits=4")
     assert d("mtx", 4, 1, 3, 8192, 22016, 128).startswith("skinny_kernel")          # long K: the few-row kernel
+    assert d("mtx", 4, 1, 2, 8192, 22016, 128).startswith("matvec_kernel<bits=4,dense,lane_groups=2,prefetch=1,rows=2> strips=172 splits=4")
+    assert d("mtx", 4, 1, 2, 14336, 4096, 128).startswith("skinny_kernel")          # ... two rows too when K is split ten ways
     assert d("mtx", 4, 1, 3, 2048, 32768, 128).startswith("skinny_kernel")          # short K: only two rows
     assert d("mtx", 4, 1, 2, 2048, 32768, 128).startswith("matvec_kernel")
     assert d("mtx", 4, 1, 5, K, S, 128).startswith("skinny_kernel")
