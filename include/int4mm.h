@@ -39,7 +39,10 @@
  * per weight: they accumulate sum(x * q) and sum(x) in fp32 and apply scale and zero
  * once per group, y += s * (sum(x * q) - z * sum(x)), which is the exact value of
  * sum(x * (q - z) * s) up to fp32 rounding -- closer to the true product than the
- * reference's fp16(fp16(q - z) * s) weights, but not the same bits.  Results are a
+ * reference's fp16(fp16(q - z) * s) weights, but not the same bits.  A single row through
+ * int4mm_matmul is served by the matvec kernel as well (overwriting outs, as the matmul
+ * does): bit for bit int4mm_matvec's result on zeroed outs, as long as the workspace holds
+ * the matvec's part (int4mm_workspace_bytes); without it a tile kernel takes the row.  Results are a
  * deterministic function of the inputs and the shape (no atomics on data).
  */
 #ifndef INT4MM_H

@@ -122,6 +122,10 @@ bool skinny_rows(int bits, _Float16* outs, const uint32_t* matrix, const _Float1
 bool matvec_rows(int bits, _Float16* outs, const uint32_t* matrix, const _Float16* x, const _Float16* scales,
                  const _Float16* zeros, int64_t R, int64_t K, int64_t S, int64_t group_size, bool accumulate,
                  hipStream_t st, void* workspace, size_t workspace_bytes);
+// a single row through the matmul entry (overwrites outs); *rc is the launch's result when the shape is taken
+bool matvec_one_row(int bits, _Float16* outs, const uint32_t* matrix, const uint32_t* sparse_mask, const _Float16* x,
+                    const _Float16* scales, const _Float16* zeros, int64_t K, int64_t S, int64_t group_size, hipStream_t st,
+                    void* workspace, size_t workspace_bytes, int* rc);
 // most rows the few-row path takes (beyond 96: only its kernel with shared staging, for the shapes it serves)
 constexpr int SK_WIDE_MAX_ROWS = 512;
 // bytes of partial tiles with which the few-row kernel splits K across workgroups (0: no split)

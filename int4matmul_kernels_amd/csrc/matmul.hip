@@ -1212,6 +1212,10 @@ extern "C" int int4mm_matmul(int bits, void* outs, const void* matrix, const voi
     hipStream_t st = (hipStream_t)stream;
     // 2 .. 96 rows in all (batches are contiguous, so they flatten; on suitable shapes up to 512): the few-row
     // kernels, which read every packed word once for all rows -- unless a tile-kernel variant is forced
+    if (B * M == 1 && !tuning(TUNE_NO_SKINNY) && !tuning(TUNE_MM_VARIANT) &&
+        matvec_one_row(bits, (h16*)outs, (const uint32_t*)matrix, (const uint32_t*)sparse_mask, (const h16*)multiplier,
+                       (const h16*)scales, (const h16*)zeros, K, S, g, st, workspace, workspace_bytes, &rc))
+        return rc;
     if (B * M >= 2 && B * M <= 4 && !sparse_mask && !tuning(TUNE_NO_SKINNY) && !tuning(TUNE_MM_VARIANT) &&
         matvec_rows(bits, (h16*)outs, (const uint32_t*)matrix, (const h16*)multiplier, (const h16*)scales, (const h16*)zeros,
                     B * M, K, S, g, false, st, workspace, workspace_bytes))

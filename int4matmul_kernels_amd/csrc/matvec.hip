@@ -811,7 +811,7 @@ void matvec_kernel(MatvecArgs a) {
         }
     };
     if (a.splits == 1) {
-        for_owned([&](int i, int ocol) { a.outs[ocol] = (h16)((float)a.outs[ocol] + total[i]); });
+        for_owned([&](int i, int ocol) { a.outs[ocol] = (h16)((a.accumulate ? (float)a.outs[ocol] : 0.f) + total[i]); });
         stamp(13); stamp(15);
         return;
     }
@@ -830,7 +830,7 @@ void matvec_kernel(MatvecArgs a) {
     // poisoned -- every result NaN -- until the host zero-fills it again)
     const uint32_t poisoned = __hip_atomic_load(a.sticky, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     for_owned([&](int i, int ocol) {
-        float sum = (float)a.outs[ocol];
+        float sum = a.accumulate ? (float)a.outs[ocol] : 0.f;
         bool ok = poisoned == 0;
         // slots are fetched eight at a time so that their latencies overlap; a
         // slot that is not full yet is polled again on its own
@@ -1015,6 +1015,24 @@ bool i4::matvec_rows(int bits, h16* outs, const uint32_t* matrix, const h16* x, 
     return true;
 }
 
+static int matvec_plain(int bits, void* outs, const void* matrix, const void* multiplier, const void* scales, const void* zeros,
+                        const void* sparse_mask, int64_t B, int64_t K, int64_t S, int64_t g, bool accumulate, void* workspace,
+                        size_t workspace_bytes, hipStream_t st);
+
+// A single row through the matmul entry (which overwrites outs): the matvec kernel serves it at the matvec's
+// rate, where a tile kernel would spend a 128-row tile on it (K=5120, S=20480: 79 -> 12 us; K=28672, S=8192:
+// 407 -> 27 us).  False when the matvec cannot take the shape with the workspace at hand.
+bool i4::matvec_one_row(int bits, h16* outs, const uint32_t* matrix, const uint32_t* sparse_mask, const h16* x, const h16* scales,
+                        const h16* zeros, int64_t K, int64_t S, int64_t group_size, hipStream_t st, void* workspace,
+                        size_t workspace_bytes, int* rc) {
+    if (K % 64 != 0 || S % 4 != 0 || tuning(TUNE_MV_TIMELINE)) return false;
+    const MatvecShape ms = plan_matvec(S, (int)(K / 64));
+    if (ms.upwg > MV_MAX_UNITS_WG) return false;
+    if (ms.splits > 1 && workspace_parts(workspace, workspace_bytes).slots_bytes < matvec_slots_bytes(S)) return false;
+    *rc = matvec_plain(bits, outs, matrix, x, scales, zeros, sparse_mask, 1, K, S, group_size, false, workspace, workspace_bytes, st);
+    return true;
+}
+
 static int matvec_impl(int bits, void* outs, const void* matrix, const void* multiplier,
                        const void* scales, const void* zeros, const void* sparse_mask,
                        const int4mm_shape* shape, void* workspace, size_t workspace_bytes,
@@ -1037,6 +1055,16 @@ static int matvec_impl(int bits, void* outs, const void* matrix, const void* mul
                     (const h16*)zeros, B, K, S, g, true, (hipStream_t)stream, (const uint32_t*)sparse_mask, workspace, workspace_bytes))
         return check_launch("matvec");
 
+    return matvec_plain(bits, outs, matrix, multiplier, scales, zeros, sparse_mask, B, K, S, g, true, workspace, workspace_bytes,
+                        (hipStream_t)stream);
+}
+
+// One launch of the single-row kernel per batch row; `accumulate`: add onto outs (the matvec entry) or
+// overwrite it (a single row through the matmul entry).
+static int matvec_plain(int bits, void* outs, const void* matrix, const void* multiplier, const void* scales, const void* zeros,
+                        const void* sparse_mask, int64_t B, int64_t K, int64_t S, int64_t g, bool accumulate, void* workspace,
+                        size_t workspace_bytes, hipStream_t st) {
+    const int units_total = (int)(K / 64);
     const MatvecShape ms = plan_matvec(S, units_total);
     const int lk = ms.lk, waves = ms.waves, upwg = ms.upwg, splits = ms.splits, strips = ms.strips;
     if (upwg > MV_MAX_UNITS_WG) return INT4MM_ERR_SHAPE;
@@ -1061,10 +1089,10 @@ static int matvec_impl(int bits, void* outs, const void* matrix, const void* mul
     a.sticky = splits > 1 ? reinterpret_cast<uint32_t*>(workspace_parts(workspace, workspace_bytes).counters - 8) : nullptr;
     a.spin_limit = tuning(TUNE_MV_SPIN) > 0 ? (int)tuning(TUNE_MV_SPIN) : MV_SPIN_LIMIT;
     a.rows = 1;
-    a.accumulate = 1;
+    a.accumulate = accumulate ? 1 : 0;
 
     const dim3 grid(strips, splits, 1), block(waves * WAVE);
-    hipStream_t st = (hipStream_t)stream;
+    int rc = INT4MM_OK;
     if (noting("matvec_kernel<bits=%d,%s,lane_groups=%d,prefetch=%d> strips=%d splits=%d waves=%d units_per_workgroup=%d batch=%d",
                bits, sparse_mask ? "16:32" : "dense", lk, (int)pf, strips, splits, waves, upwg, (int)B))
         return INT4MM_OK;

@@ -66,6 +66,10 @@ def test_two_to_four_rows_take_the_matvec_kernel_up_to_k_5120():
     assert d("vec", 3, 2, 1, K, S, 128).startswith("matvec_kernel<bits=3,dense,lane_groups=2,prefetch=0,rows=2>")
     assert d("mtx", 4, 2, 2, 4096, 11008, 128).startswith("matvec_kernel<bits=4,dense,lane_groups=4,prefetch=0,rows=4> strips=172 splits=4")
     assert d("mtx", 4, 1, 3, 8192, 22016, 128).startswith("skinny_kernel")          # long K: the few-row kernel
+    # a single row through the matmul entry: the matvec kernel (all formats), the same launch as the matvec entry's
+    for bits, sparse, g in ((4, False, 128), (3, False, 128), (2, False, 128), (4, True, 64)):
+        assert d("mtx", bits, 1, 1, K, S, g, sparse) == d("vec", bits, 1, 1, K, S, g, sparse)
+        assert d("mtx", bits, 1, 1, K, S, g, sparse).startswith("matvec_kernel<bits=%d," % bits)
     assert d("mtx", 4, 1, 2, 8192, 22016, 128).startswith("matvec_kernel<bits=4,dense,lane_groups=2,prefetch=1,rows=2> strips=172 splits=4")
     assert d("mtx", 4, 1, 2, 14336, 4096, 128).startswith("skinny_kernel")          # ... two rows too when K is split ten ways
     assert d("mtx", 4, 1, 3, 2048, 32768, 128).startswith("skinny_kernel")          # short K: only two rows

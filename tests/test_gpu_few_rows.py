@@ -481,3 +481,33 @@ def test_two_rows_long_k_with_prefetch(H):
     assert "prefetch=1,rows=2>" in tiles, tiles
     p = _problem(4, K=8192, S=20480, M=2, group_size=128, seed=14)
     _check(H, p, "mtx")
+
+
+@pytest.mark.parametrize("bits,sparse,K,S,g", [(4, False, 5120, 20480, 128), (3, False, 4096, 6144, 64), (2, False, 2048, 4096, -1),
+                                                (4, True, 4096, 8192, 64), (4, False, 128, 128, 128)])
+def test_one_row_through_the_matmul_entry(H, bits, sparse, K, S, g):
+    """a single row through the matmul entry runs the matvec kernel and overwrites outs: bit for bit the matvec
+    entry's result on zeroed outs; a column in exponent mode included.  Without a workspace, where the matvec
+    would need one, a tile kernel serves it as before."""
+    capi = H.capi
+    line = capi.describe_launch("mtx", bits, 1, 1, K, S, g, sparse)
+    assert line.startswith("matvec_kernel<"), line
+    p = _problem(bits, K=K, S=S, M=1, group_size=g, sparse=sparse, seed=K + bits)
+    p["scales"][:, 5] = -p["scales"][:, 5]
+    d = H.dev_problem(p)
+    exact, f32 = H.oracles(p)
+    ws = capi.new_matmul_workspace(1, 1, K, S, sparse)
+    args = (d["matrix"], d["states"], d["scales"], d["zeros"], g, d["mask"])
+    via_vec = torch.zeros((1, 1, S), dtype=torch.float16, device="cuda")
+    capi.matvec(bits, via_vec, *args, ws)
+    for _ in range(2):
+        via_mtx = torch.full((1, 1, S), -77.0, dtype=torch.float16, device="cuda")
+        capi.matmul(bits, via_mtx, *args, ws)
+        torch.cuda.synchronize()
+        capi.workspace_status(ws)
+        assert torch.equal(via_mtx, via_vec)
+    H.assert_product_close(via_mtx.cpu().numpy(), exact, f32, kind="vec")
+    no_ws = torch.full((1, 1, S), -77.0, dtype=torch.float16, device="cuda")
+    capi.matmul(bits, no_ws, *args, None)
+    torch.cuda.synchronize()
+    H.assert_product_close(no_ws.cpu().numpy(), exact, f32, kind="vec")

@@ -60,7 +60,8 @@ def test_matvec_exponent_mode_columns(H, bits, sparse):
     exact, f32 = H.oracles(p)
     for kind in ("vec", "mtx"):
         got = H.run_capi(p, d, kind)
-        H.assert_product_close(got, exact, f32, kind=kind)
+        # (a single row through the matmul entry is served by the matvec kernel: the matvec's class)
+        H.assert_product_close(got, exact, f32, kind="vec" if kind == "vec" else H.matmul_kind(p))
 
 
 @pytest.mark.parametrize("bits,sparse,K", [(4, False, 5120), (3, False, 1024), (2, False, 2048),

@@ -4,7 +4,8 @@ the matvec kernel and its two- / four-row forms, the few-row kernels with their 
 padded and split tiles, whole tiles.  A sweep over the row count crosses every one of those borders at
 the shapes the library is measured on; each count is checked against the float64 product on the
 oracle's fp16 weights (a library fp64 GEMM on the GPU, from the matrix the CPU oracle decoded), to the
-same bars as the other product tests, and the rows behind the last one must stay untouched."""
+same bars as the other product tests; the outputs start as NaN (the matmul entry overwrites them, with one
+row as with many), and the rows behind the last one must stay untouched."""
 import numpy as np
 import pytest
 import torch
@@ -50,8 +51,6 @@ def test_every_row_count(bits, K, S, g, sparse):
         kind = "vec" if line.startswith(("skinny_kernel", "matvec_kernel")) else "mtx"
         buf.fill_(sentinel.item())
         outs = buf[:M * S].view(1, M, S)
-        if M == 1:
-            outs.zero_()                                     # one row is the matvec, which adds onto outs
         x = states[:M].reshape(1, M, K).contiguous()
         ws = capi.new_matmul_workspace(1, M, K, S, sparse)
         capi.matmul(bits, outs, d["matrix"], x, d["scales"], d["zeros"], g, d["mask"], ws)
