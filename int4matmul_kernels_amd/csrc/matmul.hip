@@ -1158,9 +1158,18 @@ static void launch(MatmulArgs a, int64_t B, hipStream_t st, void* workspace, siz
             long_k_split = sp.ksplit >= 3 && a.K / 32 / sp.ksplit >= 140 && wsp.counters != nullptr &&
                            wsp.scratch_bytes >= (size_t)(sp.tiles * sp.ksplit * sp.tile_bytes);
         }
+        // (16:32 with at most 128 padded 256-row tiles: those, split along K, beat the 128-row tiles from K = 4096 on --
+        // K=S=8192, 896 rows: 182 -> 163 us; K=8192, S=10240, 640 rows: 178 -> 155; K=16384, S=7168, 800 rows: 346 -> 271;
+        // K=4096: 0 - 12 %; at K=2048 the unsplit 128-row tiles still win by 1 - 7 %)
+        bool sparse_split = false;
+        if (SPARSE && three_rows && pipe4_ok && tiles4 <= 128 && a.K >= 4096) {
+            const SplitPlan sp = plan_split(true, B, a.M, a.K, a.S);
+            sparse_split = sp.ksplit > 1 && wsp.counters != nullptr && sp.tiles <= 1024 &&
+                           wsp.scratch_bytes >= (size_t)(sp.tiles * sp.ksplit * sp.tile_bytes);
+        }
         if (!SPARSE && tiles4 <= 128 && a.K <= 1024) variant = 1;
         else if (long_k_split) variant = 5;
-        else if (three_rows) variant = 7;
+        else if (three_rows && !sparse_split) variant = 7;
         else if (pipe4_ok && (SPARSE || !pipe2_ok || !small_better)) variant = 6;
         else if (pipe2_ok) variant = 5;
         else if (a.M > 512 && a.S >= 256) variant = 3;

@@ -175,3 +175,20 @@ def test_tail_split_matches_oracle_and_unsplit(H, bits, sparse, M, K, S, g):
     assert O.max_rel_error(ref.astype(np.float64), runs[0]) < H.TOL_EXACT
     # the tiles that were not split are bit-identical to the plain run's
     assert np.array_equal(ref[:, :256, :256], runs[0][:, :256, :256])
+
+
+def test_sparse_odd_tile_rows_take_split_large_tiles_on_a_long_k(H):
+    """16:32, 896 rows (seven tile rows of 128) against K=4096, S=8192: 128 padded 256-row tiles split in two along K
+    instead of 224 tiles of 128 rows; without a workspace for the partial tiles the 128-row tiles as before"""
+    capi = H.capi
+    M, K, S = 896, 4096, 8192
+    assert "tile=256x256,plain> tiles=128 ksplit=2" in capi.describe_launch("mtx", 4, 1, M, K, S, 64, True)
+    assert "tile=128x256" in capi.describe_launch("mtx", 4, 1, M, K, S, 64, True, workspace_bytes=0)
+    assert "tile=128x256" in capi.describe_launch("mtx", 4, 1, M, 2048, S, 64, True)
+    p = _problem(4, True, K=K, S=S, M=M, group_size=64, seed=17)
+    p["scales"][7, 100:104] *= np.float16(-1)
+    d = H.dev_problem(p)
+    exact, f32 = H.oracles(p)
+    junk = np.full((1, M, S), 9.0, np.float16)
+    for _ in range(2):
+        H.assert_product_close(H.run_capi(p, d, "mtx", outs_init=junk), exact, f32, kind="mtx")
