@@ -1072,14 +1072,21 @@ static SplitPlan plan_split(bool sparse, int64_t B, int64_t M, int64_t K, int64_
 
 // ---- split of the last round.  256 x 256 tiles run one per CU, in rounds of 256; when the last round
 // would fill at most half of the GPU, its tiles -- and only they -- are split along K over as many
-// workgroups as fit the GPU once (at least 16 K steps each).
+// workgroups as fit half of the GPU (at least two per tile, at least 32 K steps each).
 struct TailPlan { int ksplit; int64_t split_from, tiles; };
 static TailPlan plan_tail(int64_t B, int64_t M, int64_t K, int64_t S) {
     const TailPlan none{1, 0, 0};
     if (B != 1 || S % 256 != 0 || tuning(TUNE_MM_TAIL) == 1) return none;
     const int64_t total = (M + 255) / 256 * (S / 256), tail = total % 256;
     if (total <= 256 || tail == 0 || tail > 128) return none;
-    const int64_t ks = std::min<int64_t>({256 / tail, 8, K / 32 / 16});
+    // (measured, K = 2048 ... 8192, tails of 16 ... 128 tiles: the split pays while its workgroups fill at most half of
+    // the GPU -- two per tile from 64 tiles on, where the second adds the first one's partial tile to its registers
+    // and nothing else is read back -- and while a share keeps 32 K steps: K=4096, S=8192, 2304 rows, 32 tiles in
+    // the tail: eight ways 197 us, four ways 170; K=2048, S=8192, 2560 rows, 64 tiles: four ways 121, two ways 101,
+    // unsplit 107; a tail of 97 ... 128 tiles on K = 2048 is better left whole, 110 against 117)
+    if (tail > 96 && K < 3072) return none;
+    const int64_t cap = tuning(TUNE_MM_TAIL) >= 2 ? tuning(TUNE_MM_TAIL) : 8;
+    const int64_t ks = std::min<int64_t>({std::max<int64_t>(2, 128 / tail), cap, K / 32 / 32});
     if (ks < 2 || tail * ks * (256 * 256 * 4) > MM_SPLIT_MAX_BYTES) return none;
     return TailPlan{(int)ks, total - tail, tail};
 }

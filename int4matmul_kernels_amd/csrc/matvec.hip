@@ -971,6 +971,12 @@ bool i4::matvec_rows(int bits, h16* outs, const uint32_t* matrix, const h16* x, 
     // workgroup weighs more; below K = 4096 only two rows gain.  Two rows (NR = 2) gain on a longer K as well
     // while K is split at most five ways (K=8192, S=22016: 21.0 against 26.0 us; K=28672, S=8192: 26.6 against
     // 33.3; ten splits, K=14336, S=4096: 15.5 against 13.3)
+    // Narrow outputs lose (two rows against the few-row kernel, us: K=4096, S=2048 15.1 / 9.5; K=S=4096 11.7 / 9.4;
+    // K=5120, S=6144 11.1 / 10.4; from S = 8192 on 9.3 - 10.0 / 9.6 - 10.6 and better; three and four rows: S = 6144
+    // 13 - 16 / 10, S = 8192 12 - 14 / 10, S = 11008 11.5 - 13.5 / 12.8 - 14.7), and at exactly 16384 columns the
+    // few-row kernel has one workgroup on every CU and wins for three and four rows (12.0 - 13.8 / 11.5 - 12.7)
+    if (S < 8192) return false;
+    if (R > 2 && (S < 10240 || S == 16384)) return false;
     if (R > 2 && (K > 5120 || K < 4096)) return false;
     const int units_total = (int)(K / 64);
     const MatvecShape ms = plan_matvec(S, units_total);

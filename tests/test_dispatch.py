@@ -66,6 +66,12 @@ def test_two_to_four_rows_take_the_matvec_kernel_up_to_k_5120():
     assert d("vec", 3, 2, 1, K, S, 128).startswith("matvec_kernel<bits=3,dense,lane_groups=2,prefetch=0,rows=2>")
     assert d("mtx", 4, 2, 2, 4096, 11008, 128).startswith("matvec_kernel<bits=4,dense,lane_groups=4,prefetch=0,rows=4> strips=172 splits=4")
     assert d("mtx", 4, 1, 3, 8192, 22016, 128).startswith("skinny_kernel")          # long K: the few-row kernel
+    # narrow outputs stay with the few-row kernel: two rows below 8192 columns, three and four below 10240 and at 16384
+    assert d("mtx", 4, 1, 2, 4096, 4096, 128).startswith("skinny_kernel")
+    assert d("mtx", 4, 1, 2, 4096, 8192, 128).startswith("matvec_kernel<bits=4,dense,lane_groups=4,prefetch=0,rows=2>")
+    assert d("mtx", 4, 1, 4, 5120, 8192, 128).startswith("skinny_kernel")
+    assert d("mtx", 4, 1, 4, 5120, 16384, 128).startswith("skinny_kernel")
+    assert d("mtx", 4, 1, 2, 5120, 16384, 128).startswith("matvec_kernel")
     # a single row through the matmul entry: the matvec kernel (all formats), the same launch as the matvec entry's
     for bits, sparse, g in ((4, False, 128), (3, False, 128), (2, False, 128), (4, True, 64)):
         assert d("mtx", bits, 1, 1, K, S, g, sparse) == d("vec", bits, 1, 1, K, S, g, sparse)
@@ -100,7 +106,13 @@ def test_few_rows_and_batches():
     assert d("mtx", 4, 1, 192, K, S, 128).startswith("matmul_kernel_pipe<bits=4,dense,tile=256x128")
     assert d("mtx", 4, 1, 192, 8192, 8192, 64, sparse=True).startswith("wide_rows_kernel<bits=4,16:32,row_tiles=6> strips=32 row_blocks=2 ksplit=4")
     # up to 512 rows on outputs of at most 8192 columns; wider outputs and the 16:32 format go to the tile kernels
-    assert d("mtx", 4, 1, 384, 4096, 4096, 128).startswith("wide_rows_kernel<bits=4,dense,row_tiles=4> strips=16 row_blocks=6 ksplit=2")
+    assert d("mtx", 4, 1, 384, 4096, 4096, 128).startswith("wide_rows_kernel<bits=4,dense,row_tiles=3> strips=16 row_blocks=8 ksplit=2")
+    # (65 ... 512 rows against 4096 ... 8192 columns: block height and split from the fitted cost model -- a short K is
+    # not split into shares of a few units, blocks of 48 rows where they fill the GPU better)
+    assert d("mtx", 4, 1, 416, 2048, 8192, 128).startswith("wide_rows_kernel<bits=4,dense,row_tiles=4> strips=32 row_blocks=7 ksplit=1")
+    assert d("mtx", 4, 1, 160, 4096, 8192, 128).startswith("wide_rows_kernel<bits=4,dense,row_tiles=3> strips=32 row_blocks=4 ksplit=2")
+    assert d("mtx", 3, 1, 352, 8192, 8192, 128).startswith("wide_rows_kernel<bits=3,dense,row_tiles=6> strips=32 row_blocks=4 ksplit=2")
+    assert d("mtx", 4, 1, 128, 8192, 8192, 128).startswith("wide_rows_kernel<bits=4,dense,row_tiles=4> strips=32 row_blocks=2 ksplit=4")
     assert d("mtx", 4, 1, 384, K, S, 128).startswith("matmul_kernel_pipe<bits=4,dense,tile=128x256")
     assert d("mtx", 4, 1, 384, 8192, 8192, 64, sparse=True).startswith("matmul_kernel_pipe<bits=4,16:32")
     assert d("mtx", 4, 1, 513, 4096, 4096, 128).startswith("matmul_kernel")

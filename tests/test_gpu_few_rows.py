@@ -429,10 +429,11 @@ def test_many_batch_elements_through_the_matvec_entry(H, bits, sparse):
     _check(H, p, "vec", prior=prior)
 
 
-# ---- two to four rows through the matvec kernel (a row of states per MFMA result register; dense formats, K <= 5120)
+# ---- two to four rows through the matvec kernel (a row of states per MFMA result register; dense formats, K <= 5120,
+# outputs of 8192 columns and more -- three and four rows: 10240 and more)
 @pytest.mark.parametrize("bits", [4, 3, 2])
 @pytest.mark.parametrize("R", [2, 3, 4])
-@pytest.mark.parametrize("K,S,g", [(4096, 5120, 128), (5120, 8192, 64), (4096, 6144, -1)])
+@pytest.mark.parametrize("K,S,g", [(4096, 11008, 128), (5120, 10240, 64), (4096, 12288, -1)])
 def test_two_to_four_rows_equal_the_matvec_row_by_row(H, bits, R, K, S, g):
     """the matmul entry (overwrites outs) and the matvec entry with R batch elements (adds onto outs) give, bit for
     bit, what R calls of the one-row matvec give; exponent-mode columns included"""
@@ -440,9 +441,14 @@ def test_two_to_four_rows_equal_the_matvec_row_by_row(H, bits, R, K, S, g):
     assert "rows=" in capi.describe_launch("mtx", bits, 1, R, K, S, g)
     assert "rows=" in capi.describe_launch("vec", bits, R, 1, K, S, g)
     p = _problem(bits, K=K, S=S, M=R, group_size=g, seed=R + K + S)
-    sc = p["scales"].reshape(-1, S)
+    sc, ze = p["scales"].reshape(-1, S), p["zeros"].reshape(-1, S)
     sc[0, 8:12] *= np.float16(-1)
     sc[-1, S - 1] *= np.float16(-1)
+    # (exponent-mode weights are fp16(z -+ s 2^e), rounded once per weight by the reference and the oracle, while the
+    # matvec adds z sum(x) in fp32: with z near 15 that rounding alone is worth 6e-3 of an output -- a small z keeps
+    # the comparison about the kernel)
+    ze[0, 8:12] = np.float16(0.25)
+    ze[-1, S - 1] = np.float16(0.25)
     d = H.dev_problem(p)
     exact, f32 = H.oracles(p)
     got = H.run_capi(p, d, "mtx", outs_init=np.full((1, R, S), 7.0, np.float16))

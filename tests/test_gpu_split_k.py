@@ -145,8 +145,8 @@ def test_extension_workspace_survives_changing_shapes(H):
 # ---- grids of 256 x 256 tiles whose last round of 256 fills at most half of the GPU: only the tiles of
 # that round are split along K (tuning key 7 = 1 switches it off)
 @pytest.mark.parametrize("bits,sparse", FORMATS)
-@pytest.mark.parametrize("M,K,S,g", [(512, 1024, 33280, 128),        # 260 tiles: 4 split in two
-                                     (2200, 2048, 7424, 64)])        # 261 tiles: 5 split in four
+@pytest.mark.parametrize("M,K,S,g", [(512, 2048, 33280, 128),        # 260 tiles: 4 split in two (shares of 32 K steps)
+                                     (2200, 4096, 7424, 64)])        # 261 tiles: 5 split in four
 def test_tail_split_matches_oracle_and_unsplit(H, bits, sparse, M, K, S, g):
     capi = H.capi
     p = _problem(bits, sparse, K=K, S=S, M=M, group_size=g, seed=M + K + 1)
