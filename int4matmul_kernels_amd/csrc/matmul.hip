@@ -1134,11 +1134,13 @@ static void launch(MatmulArgs a, int64_t B, hipStream_t st, void* workspace, siz
     // they give the GPU at most one round of at least half (16:32: three quarters) of its CUs; smaller grids
     // are better off with split-K
     const int64_t rows_128 = (a.M + 127) / 128, tiles_128 = rows_128 * (a.S / 256) * B;
-    // (dense: also with an even number of rows when the 128 x 256 tiles fill five eighths of the GPU and more --
+    // (dense: also with an even number of rows when the 128 x 256 tiles fill nine sixteenths of the GPU and more --
     // better than half as many 256 x 256 tiles or 256 x 128 tiles with split-K, by 5 - 10 %)
-    const bool odd_rows = rows_128 % 2 == 1 && rows_128 <= 9;
+    // (K=S=3072, eleven to thirteen rows of 128: 132 - 156 tiles of 128 x 256 in 49 - 50 us against 56 - 59 for the
+    // 256 x 128 tiles that used to serve 1408 ... 1664 rows there)
+    const bool odd_rows = rows_128 % 2 == 1 && rows_128 <= (SPARSE ? 9 : 13);
     const bool three_rows = a.M > 256 && shape_ok && a.S % 256 == 0 && tiles_128 <= 256 &&
-                            (SPARSE ? odd_rows && tiles_128 >= 192 : tiles_128 >= (odd_rows ? 128 : 160));
+                            (SPARSE ? odd_rows && tiles_128 >= 192 : tiles_128 >= (odd_rows ? 128 : 144));
     const bool pipe2_ok = !SPARSE && m_ok && a.S % 128 == 0;
     const bool pipe4_ok = m_ok && a.S % 256 == 0;
     if (variant != 1 && variant != 3 && variant != 5 && variant != 6 && variant != 7 && variant != 9) variant = 0;

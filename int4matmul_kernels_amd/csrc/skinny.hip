@@ -916,6 +916,19 @@ static int64_t wide_groups(int64_t units, int64_t units_per_split, int64_t kspli
 constexpr size_t WIDE_LDS_LIMIT = 150 * 1024;
 
 // `group_units`: 64-row units per quantisation group (K / 64 and more: a single group)
+// Whether the few-row kernel above runs 33 ... 96 rows (two or three row blocks per strip) as one round of 128 ... 256
+// workgroups, or through its own split-K on a narrow output (the same conditions as unsplit_cw / plan_skinny_split).
+static bool skinny_one_round(int64_t R, int64_t S, bool sparse) {
+    const int64_t blocks = (R + 31) / 32;
+    if (S % 64 == 0 && S / 32 * blocks < 192) return true;
+    for (const int c : {4, 2, 1}) {
+        if (sparse && c == 4) continue;
+        const int64_t wgs = S / (16 * c) * blocks;
+        if (S % (16 * c) == 0 && wgs >= 128 && wgs <= 256) return true;
+    }
+    return false;
+}
+
 static WidePlan plan_wide(int64_t R, int64_t K, int64_t S, bool sparse, int64_t group_units) {
     WidePlan p{false, 0, 0, 0, 1, 0, 0};
     // (knob: 1 = never, n >= 2 = from n rows on whatever the shape)
@@ -957,14 +970,15 @@ static WidePlan plan_wide(int64_t R, int64_t K, int64_t S, bool sparse, int64_t 
     };
     shape(128);
     if (R <= 64 || ks > 6 || (ks > 1 && units / ks < 20)) shape(64);
-    // 65 ... 512 rows of a dense format against 4096 ... 8192 columns, where this kernel always serves: block height
+    // 65 ... 512 rows of a dense format against 2048 ... 8192 columns, where this kernel always serves: block height
     // (up to 128, 96, 64 or 48 rows) and split by a cost model fitted to 4 900 timed launches (int4, K = 2048 ...
-    // 28672, 72 ... 512 rows; its pick is within 0.3 % of the best measured candidate on average, 6.6 % at worst,
+    // 28672, S = 4096 ... 8192, 72 ... 512 rows; its pick is within 0.3 % of the best measured candidate on average,
+    // 6.6 % at worst -- on 1 800 more launches at S = 2048 and 3072 with up to 16 splits, not used in the fit: 0.3 / 3.8 % --,
     // where the rules above were 8 % off on K <= 8192 and up to 73 % -- e.g. K=2048, S=8192, 416 rows: seven blocks
     // of 64 rows split four ways, 49 us, against 28 us unsplit; int3, int2 and other group sizes rank alike):
     // a workgroup takes a[row tiles] us per 64-row unit of its share plus 3.9 us; a split costs 0.8 us per way
     // and 1.9 us per row tile, less 4.2; workgroups run in rounds of 256, the last one charged 3.5 us x its fill.
-    if (!sparse && R > 64 && S >= 4096 && S <= 8192 && forced < 1) {
+    if (!sparse && R > 64 && S >= 2048 && S <= 8192 && forced < 1) {
         static const double per_unit[9] = {0, 0, 0, 0.617, 0.707, 0, 0.912, 0, 1.059};
         const size_t room = WIDE_LDS_LIMIT;
         double best = 1e30;
@@ -972,7 +986,7 @@ static WidePlan plan_wide(int64_t R, int64_t K, int64_t S, bool sparse, int64_t 
         for (const int64_t tallest : {128, 96, 64, 48}) {
             shape(tallest);
             const int64_t tiles = wgs;
-            for (int64_t k = 1; k <= 8 && (k == 1 || units / k >= 8) && tiles * k <= 1024; ++k) {
+            for (int64_t k = 1; k <= 16 && (k == 1 || units / k >= 8) && tiles * k <= 1024; ++k) {
                 const int64_t share = (units + k - 1) / k, rounds = (tiles * k + 255) / 256, last = tiles * k - (rounds - 1) * 256;
                 if (wide_lds_bytes(p.block_rows, wide_groups(units, share, (units + share - 1) / share, group_units)) > room) continue;
                 const double t = rounds * (per_unit[p.mt] * share + 3.92) + (k > 1 ? -4.164 + 0.798 * k + 1.915 * p.mt : 0.0) +
@@ -1004,7 +1018,14 @@ static WidePlan plan_wide(int64_t R, int64_t K, int64_t S, bool sparse, int64_t 
             if (R > 128 && (S > 8192 || (R > 256 && S > 4096))) return p;
         } else {
             if (R <= 32 && (wgs < 32 || wgs > 96 || p.units_per_split < 16)) return p;
-            if (R > 32 && R <= 64 && K * S < (1ll << 25)) return p;
+            // (33 ... 64 rows are two row blocks of the kernel above: where its strips can be cut to give one round of
+            // 128 ... 256 workgroups -- or its own split-K serves a narrow output -- it wins up to K = 5120, on outputs
+            // of at most 4096 columns up to K = 8192 and below 3072 columns always: K=S=4096, 40 / 64 rows 13.0 / 13.2
+            // against 16.1 / 18.7 us; K=5120, S=8192 18.5 / 18.9 against 19.4 / 22.3; K=8192, S=4096 19.5 / 19.6 against
+            // 22.3 / 26.6; K=8192, S=6144 24.7 / 25.0 against 21.9 / 25.4; K=14336, S=5120 36.9 against 27.6 / 31.3)
+            if (R > 32 && R <= 64 &&
+                (skinny_one_round(R, S, false) ? (K <= 5120 || (K <= 8192 && S <= 4096) || S < 3072) : K * S < (1ll << 25)))
+                return p;
             // (beyond 8192 columns only in row blocks of 96 / 128 rows: K=2048, S=12288, 192 rows in three blocks of
             // 64: 37 against 32 us)
             if (R > 128 && S > 8192 && (S > (R <= 192 ? 14336 : R <= 256 ? 10240 : 8192) || p.block_rows <= 64)) return p;
@@ -1089,6 +1110,19 @@ static bool launch_skinny_cw(const SkinnyArgs& a, int cw, int waves, int ksplit,
 // least 256 workgroups, else at least 128 (narrow strips use half a cache line per packed row).
 static int unsplit_cw(int64_t R, int64_t S, bool sparse) {
     int cw = 1;
+    // (more than 32 rows run as two or three row blocks per strip, each a workgroup: the widest strips -- within what
+    // the format's registers allow -- that give one round of 128 ... 256 workgroups, where there are such: K=2048,
+    // S=8192, 40 rows in 256 workgroups of 64 columns instead of 512 of 32)
+    if (R > 32) {
+        const int64_t blocks = (R + 31) / 32;
+        int64_t best = 0;
+        for (const int c : {4, 2, 1}) {
+            if (sparse && c == 4) continue;
+            const int64_t wgs = S / (16 * c) * blocks;
+            if (S % (16 * c) == 0 && wgs >= 128 && wgs <= 256 && wgs > best) { best = wgs; cw = c; }
+        }
+        if (best != 0) return cw;
+    }
     const int prefer[4][2] = {{4, 256}, {2, 256}, {4, 128}, {2, 128}};       // {columns per lane, workgroups}
     for (const auto& c : prefer)
         if (S % (16 * c[0]) == 0 && S / (16 * c[0]) >= c[1]) { cw = c[0]; break; }
