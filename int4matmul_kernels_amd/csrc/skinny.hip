@@ -1012,7 +1012,13 @@ static WidePlan plan_wide(int64_t R, int64_t K, int64_t S, bool sparse, int64_t 
     if (knob < 2 && forced < 1) {
         if (sparse) {
             if (R <= 32 && K * S < (1ll << 26)) return p;
-            if (R > 32 && R <= 64 && K * S < (1ll << 25)) return p;
+            // (33 ... 64 rows: the kernel above while its two row blocks per strip make one round of workgroups -- outputs
+            // of at most 4096 columns -- up to K = 8192: K=S=4096, 40 / 64 rows 16.3 / 16.3 against 20.9 / 23.4 us; K=8192,
+            // S=4096 25.3 / 24.8 against 27.5 / 31.1; beyond that only on a short K: K=4096, S=5120 28.3 / 29.3 against
+            // 22.5 / 24.8; K=5120, S=6144 33.5 / 33.9 against 23.3 / 26.7)
+            if (R > 32 && R <= 64 &&
+                (skinny_one_round(R, S, true) ? (K <= 8192 || S < 3072) : (K < 4096 && K * S < (1ll << 25))))
+                return p;
             // (the padded 256-row tiles win on very wide outputs against two row blocks)
             if (R > 96 && R <= 128 && S > 16384 && p.row_blocks > 1) return p;
             if (R > 128 && (S > 8192 || (R > 256 && S > 4096))) return p;
