@@ -82,7 +82,7 @@ INT4MM_API int int4mm_abi_version(void);
 /* Benchmark / tuning hook, not part of the drop-in boundary: overrides a launch
  * heuristic for the calling host thread (value 0 restores the default).  key 0 = waves per
  * workgroup of the matvec and few-row kernels, 1 = matvec 64-row units per lane
- * group, 2 = matvec lane groups per wave (1, 2, 4), 3 = matmul kernel variant
+ * group, 2 = matvec lane groups per wave / few-row kernel columns per lane (1, 2, 4), 3 = matmul kernel variant
  * (5 / 6 / 7 = pipelined 256x128 / 256x256 / 128x256 tiles, 9 = 256x256 without
  * the two-phase order; a forced variant also keeps the product away from the
  * few-row kernels), 4 = matvec: 1 disables prefetch,

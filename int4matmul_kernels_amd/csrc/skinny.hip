@@ -1024,6 +1024,10 @@ static WidePlan plan_wide(int64_t R, int64_t K, int64_t S, bool sparse, int64_t 
             if (R > 128 && (S > 8192 || (R > 256 && S > 4096))) return p;
         } else {
             if (R <= 32 && (wgs < 32 || wgs > 96 || p.units_per_split < 16)) return p;
+            // (one round of 129 ... 256 strips of 64 columns: the kernel above up to K = 6144 -- K=4096, S=14336, 20 / 32
+            // rows 16.3 / 17.7 against 18.4 / 18.3 us; K=5120, S=16384 19.4 / 21.8 against 22.7 / 22.8; K=8192, S=12288
+            // 25.8 / 27.1 against 25.1 / 25.1)
+            if (R <= 32 && S % 64 == 0 && S / 64 > 128 && S / 64 <= 256 && K <= 6144) return p;
             // (33 ... 64 rows are two row blocks of the kernel above: where its strips can be cut to give one round of
             // 128 ... 256 workgroups -- or its own split-K serves a narrow output -- it wins up to K = 5120, on outputs
             // of at most 4096 columns up to K = 8192 and below 3072 columns always: K=S=4096, 40 / 64 rows 13.0 / 13.2
@@ -1129,7 +1133,10 @@ static int unsplit_cw(int64_t R, int64_t S, bool sparse) {
         }
         if (best != 0) return cw;
     }
-    const int prefer[4][2] = {{4, 256}, {2, 256}, {4, 128}, {2, 128}};       // {columns per lane, workgroups}
+    // (64-column strips as soon as they give more than half a round of workgroups: 129 ... 255 of them finish in one
+    // round where twice as many 32-column strips need two -- up to 16 rows, us: K=8192, S=12288 21.5 -> 17.4; K=14336,
+    // S=14336 38.3 -> 25.5; K=4096, S=10240 12.9 -> 11.9; 16:32, K=8192, S=12288 32.8 -> 26.0)
+    const int prefer[4][2] = {{4, 129}, {2, 256}, {4, 128}, {2, 128}};       // {columns per lane, workgroups}
     for (const auto& c : prefer)
         if (S % (16 * c[0]) == 0 && S / (16 * c[0]) >= c[1]) { cw = c[0]; break; }
     // (16:32 with more than 16 rows: four columns per lane would not fit the register file)
@@ -1209,6 +1216,11 @@ bool skinny_rows(int bits, h16* outs, const uint32_t* matrix, const h16* x, cons
     // workgroup per CU, where eight waves keep twice the bytes in flight (K=5120, S=16384, 8 rows:
     // 14.6 -> 12.0 us; K=S=8192: 16.5 -> 12.3 us; 320 and 448 strips: 17.7 against 22.2, 27 against 32)
     int cw = unsplit_cw(R, S, sparse_mask != nullptr);
+    {   // (tuning: columns per lane of the few-row kernel where the shape allows them)
+        const int64_t forced_cw = tuning(TUNE_MV_LK);
+        if ((forced_cw == 1 || forced_cw == 2 || (forced_cw == 4 && !(sparse_mask && R > 16))) && S % (16 * forced_cw) == 0)
+            cw = (int)forced_cw;
+    }
     const int units = (int)(K / 64);
     int waves = (int)tuning(TUNE_MV_WAVES);
     if (waves != 2 && waves != 4 && waves != 8) waves = S / (16 * cw) > 256 && units < 160 ? 4 : 8;
