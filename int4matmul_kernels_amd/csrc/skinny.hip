@@ -970,6 +970,9 @@ static WidePlan plan_wide(int64_t R, int64_t K, int64_t S, bool sparse, int64_t 
     };
     shape(128);
     if (R <= 64 || ks > 6 || (ks > 1 && units / ks < 20)) shape(64);
+    // (49 ... 64 rows on a narrow output: two blocks of 32 rows with half the splits instead of one block of 64 --
+    // K=11008, S=4096: 28.7 -> 23.0 us; K=14336, S=4096: 31.3 -> 26.9; from 5120 columns on the single block wins on a long K)
+    if (!sparse && R > 48 && R <= 64 && S <= 4096 && forced < 1) shape(32);
     // 65 ... 512 rows of a dense format against 2048 ... 8192 columns, where this kernel always serves: block height
     // (up to 128, 96, 64 or 48 rows) and split by a cost model fitted to 4 900 timed launches (int4, K = 2048 ...
     // 28672, S = 4096 ... 8192, 72 ... 512 rows; its pick is within 0.3 % of the best measured candidate on average,

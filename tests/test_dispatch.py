@@ -122,6 +122,7 @@ def test_few_rows_and_batches():
     assert d("mtx", 4, 1, 40, 2048, 8192, 128).startswith("skinny_kernel<bits=4,dense,columns_per_lane=4,row_tiles=4> strips=128 row_blocks=2")
     assert d("mtx", 4, 1, 64, 8192, 4096, 128).startswith("skinny_kernel<bits=4,dense,columns_per_lane=2,row_tiles=4> strips=128 row_blocks=2")
     assert d("mtx", 4, 1, 64, 8192, 8192, 128).startswith("wide_rows_kernel<bits=4,dense,row_tiles=4>")
+    assert d("mtx", 4, 1, 64, 11008, 4096, 128).startswith("wide_rows_kernel<bits=4,dense,row_tiles=2> strips=16 row_blocks=2 ksplit=8")
     assert d("mtx", 4, 1, 40, 4096, 5120, 64, True).startswith("wide_rows_kernel<bits=4,16:32,row_tiles=3>")
     assert d("mtx", 4, 1, 40, 8192, 4096, 64, True).startswith("skinny_kernel<bits=4,16:32,columns_per_lane=2,row_tiles=4> strips=128 row_blocks=2")
     assert d("mtx", 4, 1, 257, K, S, 128).startswith("matmul_kernel_pipe<bits=4,dense,tile=128x256")

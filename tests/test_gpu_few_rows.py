@@ -517,3 +517,20 @@ def test_one_row_through_the_matmul_entry(H, bits, sparse, K, S, g):
     capi.matmul(bits, no_ws, *args, None)
     torch.cuda.synchronize()
     H.assert_product_close(no_ws.cpu().numpy(), exact, f32, kind="vec")
+
+
+@pytest.mark.parametrize("bits", [4, 3])
+def test_two_row_blocks_of_32_on_a_narrow_output_long_k(H, bits):
+    """49 ... 64 rows against K=11008, S=4096: the shared-staging kernel in two blocks of 32 rows, K split eight ways;
+    an exponent-mode group included"""
+    M, K, S, g = 60, 11008, 4096, 128
+    tiles = H.capi.describe_launch("mtx", bits, 1, M, K, S, g)
+    assert tiles.startswith("wide_rows_kernel<bits=%d,dense,row_tiles=2> strips=16 row_blocks=2 ksplit=8" % bits), tiles
+    p = _problem(bits, K=K, S=S, M=M, group_size=g, seed=61)
+    p["scales"][40, 1000:1004] *= np.float16(-1)
+    p["zeros"][40, 1000:1004] = np.float16(0.5)
+    d = H.dev_problem(p)
+    exact, f32 = H.oracles(p)
+    got = H.run_capi(p, d, "mtx", outs_init=np.full((1, M, S), 2.0, np.float16))
+    H.assert_product_close(got, exact, f32, kind="mtx")
+    assert np.array_equal(got, H.run_capi(p, d, "mtx"))
