@@ -1026,7 +1026,9 @@ static WidePlan plan_wide(int64_t R, int64_t K, int64_t S, bool sparse, int64_t 
             if (R > 96 && R <= 128 && S > 16384 && p.row_blocks > 1) return p;
             if (R > 128 && (S > 8192 || (R > 256 && S > 4096))) return p;
         } else {
-            if (R <= 32 && (wgs < 32 || wgs > 96 || p.units_per_split < 16)) return p;
+            // (24 ... 31 strips only on a long K: K=14336, S=6144, 20 / 32 rows 24.5 / 24.5 against 29.6 / 32.3 us for the
+            // kernel above; K=8192, S=6144 18.9 / 19.0 against 18.7 / 19.5)
+            if (R <= 32 && (wgs < (units >= 160 ? 24 : 32) || wgs > 96 || p.units_per_split < 16)) return p;
             // (one round of 129 ... 256 strips of 64 columns: the kernel above up to K = 6144 -- K=4096, S=14336, 20 / 32
             // rows 16.3 / 17.7 against 18.4 / 18.3 us; K=5120, S=16384 19.4 / 21.8 against 22.7 / 22.8; K=8192, S=12288
             // 25.8 / 27.1 against 25.1 / 25.1)
