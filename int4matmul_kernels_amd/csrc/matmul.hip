@@ -23,6 +23,7 @@
 #include "common.h"
 
 #include <algorithm>
+#include <cmath>
 #include <type_traits>
 
 namespace i4 {
@@ -1058,7 +1059,18 @@ static SplitPlan plan_split(bool sparse, int64_t B, int64_t M, int64_t K, int64_
     SplitPlan p{1, m_pad / 256 * (S / (sparse ? 256 : 128)) * B, sparse ? 256 * 256 * 4 : 256 * 128 * 4};
     if (p.tiles > MM_SPLIT_MAX_TILES) return none;
     const int64_t steps = K / 32, forced = tuning(TUNE_MM_SPLIT);
-    auto cost = [&](int64_t ks) { return (p.tiles * ks + 255) / 256 * ((steps + ks - 1) / ks + 20) + (ks > 1 ? 6 * ks : 0); };
+    // (16:32, whose 256 x 256 tiles run one per CU: a GPU filled to the last CU runs its K steps 39 % slower than a
+    // nearly empty one -- the power limit --, three quarters full 15 % slower; fitted to 320 timed launches, K = 2048 ...
+    // 14336, 16 ... 128 tiles, 1 ... 8 ways: 64 tiles at K=4096 four ways 79 us, three ways 68; 32 tiles at K=14336 eight
+    // ways 125, six ways 106.  Its pick is within 1 % of the best measured factor on average, 10 % at worst; without
+    // the term 3 % / 20 %.  The dense formats' 256 x 128 tiles, two workgroups per CU, are within 1.4 % / 11 % as is.)
+    auto cost = [&](int64_t ks) -> double {
+        const int64_t wgs = p.tiles * ks, rounds = (wgs + 255) / 256;
+        const double own = (double)(rounds * ((steps + ks - 1) / ks + 20));
+        if (!sparse) return own + (ks > 1 ? 6.0 * ks : 0.0);
+        const double fill = wgs >= 256 ? 1.0 : wgs / 256.0;
+        return own * (1.0 + 0.39 * std::pow(fill, 3.2)) + (ks > 1 ? 5.0 * ks : 0.0);
+    };
     int64_t best = 1;
     for (int64_t ks = 2; ks <= 8; ++ks) {
         if (steps / ks < 8 || p.tiles * ks * p.tile_bytes > MM_SPLIT_MAX_BYTES) break;
