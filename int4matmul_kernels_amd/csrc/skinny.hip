@@ -981,9 +981,16 @@ static WidePlan plan_wide(int64_t R, int64_t K, int64_t S, bool sparse, int64_t 
     // of 64 rows split four ways, 49 us, against 28 us unsplit; int3, int2 and other group sizes rank alike):
     // a workgroup takes a[row tiles] us per 64-row unit of its share plus 3.9 us; a split costs 0.8 us per way
     // and 1.9 us per row tile, less 4.2; workgroups run in rounds of 256, the last one charged 3.5 us x its fill.
-    if (!sparse && R > 64 && S >= 2048 && S <= 8192 && forced < 1) {
-        static const double per_unit[9] = {0, 0, 0, 0.617, 0.707, 0, 0.912, 0, 1.059};
-        const size_t room = WIDE_LDS_LIMIT;
+    // (16:32, fitted apart to 2 300 launches at S = 4096 ... 8192: 1.12 / 1.20 / 1.32 / 1.54 us per unit, 4.2 us per
+    // workgroup, a split 0.9 us per way + 1.7 per row tile - 3.7, the last round 5.3 us x its fill; the pick is within
+    // 0.1 % of the best candidate on average, 2.8 % at worst, where the rules above were 5 % / 27 % off -- K=4096,
+    // S=8192, 160 rows 50 -> 39 us; K=14336, S=8192, 128 rows 82 -> 69)
+    struct WideCost { double per_unit[9], workgroup, split, per_way, per_tile, last_round; };
+    static const WideCost dense_cost = {{0, 0, 0, 0.617, 0.707, 0, 0.912, 0, 1.059}, 3.92, -4.164, 0.798, 1.915, 3.544};
+    static const WideCost sparse_cost = {{0, 0, 0, 1.12, 1.203, 0, 1.32, 0, 1.537}, 4.17, -3.744, 0.921, 1.701, 5.284};
+    if (R > 64 && S >= (sparse ? 4096 : 2048) && S <= 8192 && forced < 1) {
+        const WideCost& wc = sparse ? sparse_cost : dense_cost;
+        const size_t room = WIDE_LDS_LIMIT - (sparse ? 4096 : 0);
         double best = 1e30;
         int64_t best_tall = 0, best_ks = 1;
         for (const int64_t tallest : {128, 96, 64, 48}) {
@@ -992,8 +999,9 @@ static WidePlan plan_wide(int64_t R, int64_t K, int64_t S, bool sparse, int64_t 
             for (int64_t k = 1; k <= 16 && (k == 1 || units / k >= 8) && tiles * k <= 1024; ++k) {
                 const int64_t share = (units + k - 1) / k, rounds = (tiles * k + 255) / 256, last = tiles * k - (rounds - 1) * 256;
                 if (wide_lds_bytes(p.block_rows, wide_groups(units, share, (units + share - 1) / share, group_units)) > room) continue;
-                const double t = rounds * (per_unit[p.mt] * share + 3.92) + (k > 1 ? -4.164 + 0.798 * k + 1.915 * p.mt : 0.0) +
-                                 (rounds > 1 ? 3.544 * last / 256.0 : 0.0);
+                const double t = rounds * (wc.per_unit[p.mt] * share + wc.workgroup) +
+                                 (k > 1 ? wc.split + wc.per_way * k + wc.per_tile * p.mt : 0.0) +
+                                 (rounds > 1 ? wc.last_round * last / 256.0 : 0.0);
                 if (t < best) { best = t; best_tall = tallest; best_ks = k; }
             }
         }

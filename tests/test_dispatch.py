@@ -98,7 +98,8 @@ def test_few_rows_and_batches():
     assert d("mtx", 4, 1, 200, 28672, 8192, 128).startswith("wide_rows_kernel<bits=4,dense,row_tiles=8> strips=32 row_blocks=2 ksplit=4")
     assert d("mtx", 4, 1, 96, K, S, 64, sparse=True).startswith("wide_rows_kernel<bits=4,16:32,row_tiles=6> strips=80 row_blocks=1 ksplit=3")
     assert d("mtx", 4, 1, 128, K, S, 64, sparse=True).startswith("wide_rows_kernel<bits=4,16:32,row_tiles=8> strips=80 row_blocks=1 ksplit=3")
-    assert d("mtx", 4, 1, 128, 8192, 8192, 64, sparse=True).startswith("wide_rows_kernel<bits=4,16:32,row_tiles=4> strips=32 row_blocks=2 ksplit=4")
+    # (16:32 against 4096 ... 8192 columns: block height and split from its own fitted cost model)
+    assert d("mtx", 4, 1, 128, 8192, 8192, 64, sparse=True).startswith("wide_rows_kernel<bits=4,16:32,row_tiles=8> strips=32 row_blocks=1 ksplit=8")
     # 129 ... 256 rows: also on wider outputs (up to 14336 / 10240 columns) in row blocks of 96 / 128 rows
     assert d("mtx", 4, 1, 192, 4096, 14336, 128).startswith("wide_rows_kernel<bits=4,dense,row_tiles=6> strips=56 row_blocks=2 ksplit=2")
     assert d("mtx", 4, 1, 256, 4096, 14336, 128).startswith("matmul_kernel_pipe<bits=4,dense,tile=256x128")
