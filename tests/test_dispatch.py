@@ -100,11 +100,14 @@ def test_few_rows_and_batches():
     assert d("mtx", 4, 1, 128, K, S, 64, sparse=True).startswith("wide_rows_kernel<bits=4,16:32,row_tiles=8> strips=80 row_blocks=1 ksplit=3")
     # (16:32 against 4096 ... 8192 columns: block height and split from its own fitted cost model)
     assert d("mtx", 4, 1, 128, 8192, 8192, 64, sparse=True).startswith("wide_rows_kernel<bits=4,16:32,row_tiles=8> strips=32 row_blocks=1 ksplit=8")
-    # 129 ... 256 rows: also on wider outputs (up to 14336 / 10240 columns) in row blocks of 96 / 128 rows
+    # 129 ... 192 rows: on any output up to 32768 columns, with the block height and split the cost model picks;
+    # 193 ... 256 rows: up to 10240 columns, and wider ones on a K of at most 4096
     assert d("mtx", 4, 1, 192, 4096, 14336, 128).startswith("wide_rows_kernel<bits=4,dense,row_tiles=6> strips=56 row_blocks=2 ksplit=2")
-    assert d("mtx", 4, 1, 256, 4096, 14336, 128).startswith("matmul_kernel_pipe<bits=4,dense,tile=256x128")
-    assert d("mtx", 4, 1, 192, 2048, 12288, 128).startswith("matmul_kernel_pipe<bits=4,dense,tile=256x128")
-    assert d("mtx", 4, 1, 192, K, S, 128).startswith("matmul_kernel_pipe<bits=4,dense,tile=256x128")
+    assert d("mtx", 4, 1, 256, 4096, 14336, 128).startswith("wide_rows_kernel<bits=4,dense,row_tiles=4> strips=56 row_blocks=4 ksplit=1")
+    assert d("mtx", 4, 1, 192, 2048, 12288, 128).startswith("wide_rows_kernel<bits=4,dense,row_tiles=3> strips=48 row_blocks=4 ksplit=1")
+    assert d("mtx", 4, 1, 192, K, S, 128).startswith("wide_rows_kernel<bits=4,dense,row_tiles=4> strips=80 row_blocks=3 ksplit=1")
+    assert d("mtx", 4, 1, 256, K, S, 128).startswith("matmul_kernel_pipe<bits=4,dense,tile=256x128")
+    assert d("mtx", 4, 1, 256, 8192, 14336, 128).startswith("matmul_kernel_pipe<bits=4,dense,tile=256x128")
     assert d("mtx", 4, 1, 192, 8192, 8192, 64, sparse=True).startswith("wide_rows_kernel<bits=4,16:32,row_tiles=6> strips=32 row_blocks=2 ksplit=4")
     # up to 512 rows on outputs of at most 8192 columns; wider outputs and the 16:32 format go to the tile kernels
     assert d("mtx", 4, 1, 384, 4096, 4096, 128).startswith("wide_rows_kernel<bits=4,dense,row_tiles=3> strips=16 row_blocks=8 ksplit=2")
