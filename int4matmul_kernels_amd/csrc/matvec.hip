@@ -976,7 +976,9 @@ bool i4::matvec_rows(int bits, h16* outs, const uint32_t* matrix, const h16* x, 
     // 13 - 16 / 10, S = 8192 12 - 14 / 10, S = 11008 11.5 - 13.5 / 12.8 - 14.7), and at exactly 16384 columns the
     // few-row kernel has one workgroup on every CU and wins for three and four rows (12.0 - 13.8 / 11.5 - 12.7)
     if (S < 8192) return false;
-    if (R > 2 && (S < 10240 || S == 16384)) return false;
+    // (... and up to 16384 columns altogether since the few-row kernel takes such outputs in one round of 64-column
+    // strips: K=4096, S=14336, three / four rows 11.4 / 12.6 against 10.3 us)
+    if (R > 2 && S <= 16384) return false;
     if (R > 2 && (K > 5120 || K < 4096)) return false;
     const int units_total = (int)(K / 64);
     const MatvecShape ms = plan_matvec(S, units_total);

@@ -64,9 +64,10 @@ def test_two_to_four_rows_take_the_matvec_kernel_up_to_k_5120():
     assert d("mtx", 4, 1, 3, K, S, 128).startswith(
         "matvec_kernel<bits=4,dense,lane_groups=2,prefetch=0,rows=4> strips=160 splits=4 waves=4 units_per_workgroup=23 rows=3")
     assert d("vec", 3, 2, 1, K, S, 128).startswith("matvec_kernel<bits=3,dense,lane_groups=2,prefetch=0,rows=2>")
-    assert d("mtx", 4, 2, 2, 4096, 11008, 128).startswith("matvec_kernel<bits=4,dense,lane_groups=4,prefetch=0,rows=4> strips=172 splits=4")
+    assert d("mtx", 4, 2, 2, 4096, 22016, 128).startswith("matvec_kernel<bits=4,dense,lane_groups=2,prefetch=0,rows=4> strips=172 splits=")
+    assert d("mtx", 4, 2, 2, 4096, 11008, 128).startswith("skinny_kernel")           # (one round of 64-column strips there)
     assert d("mtx", 4, 1, 3, 8192, 22016, 128).startswith("skinny_kernel")          # long K: the few-row kernel
-    # narrow outputs stay with the few-row kernel: two rows below 8192 columns, three and four below 10240 and at 16384
+    # narrow outputs stay with the few-row kernel: two rows below 8192 columns, three and four up to 16384
     assert d("mtx", 4, 1, 2, 4096, 4096, 128).startswith("skinny_kernel")
     assert d("mtx", 4, 1, 2, 4096, 8192, 128).startswith("matvec_kernel<bits=4,dense,lane_groups=4,prefetch=0,rows=2>")
     assert d("mtx", 4, 1, 4, 5120, 8192, 128).startswith("skinny_kernel")

@@ -430,10 +430,10 @@ def test_many_batch_elements_through_the_matvec_entry(H, bits, sparse):
 
 
 # ---- two to four rows through the matvec kernel (a row of states per MFMA result register; dense formats, K <= 5120,
-# outputs of 8192 columns and more -- three and four rows: 10240 and more)
+# outputs of 8192 columns and more -- three and four rows: more than 16384)
 @pytest.mark.parametrize("bits", [4, 3, 2])
 @pytest.mark.parametrize("R", [2, 3, 4])
-@pytest.mark.parametrize("K,S,g", [(4096, 11008, 128), (5120, 10240, 64), (4096, 12288, -1)])
+@pytest.mark.parametrize("K,S,g", [(4096, 22016, 128), (5120, 17408, 64), (4096, 18432, -1)])
 def test_two_to_four_rows_equal_the_matvec_row_by_row(H, bits, R, K, S, g):
     """the matmul entry (overwrites outs) and the matvec entry with R batch elements (adds onto outs) give, bit for
     bit, what R calls of the one-row matvec give; exponent-mode columns included"""
