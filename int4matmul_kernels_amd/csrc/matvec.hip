@@ -1063,8 +1063,25 @@ static int matvec_impl(int bits, void* outs, const void* matrix, const void* mul
                     (const h16*)zeros, B, K, S, g, true, (hipStream_t)stream, (const uint32_t*)sparse_mask, workspace, workspace_bytes))
         return check_launch("matvec");
 
-    return matvec_plain(bits, outs, matrix, multiplier, scales, zeros, sparse_mask, B, K, S, g, true, workspace, workspace_bytes,
-                        (hipStream_t)stream);
+    // more batch elements than the few-row kernels take at once: chunks of up to 512 through them (they add onto outs
+    // as the matvec does; 1 100 elements at K=4096, S=4096: three launches instead of 1 100), the plain kernel for what
+    // they do not take
+    int64_t done = 0;
+    if (B > SK_WIDE_MAX_ROWS && !tuning(TUNE_NO_SKINNY)) {
+        while (B - done >= 2) {
+            const int64_t n = std::min<int64_t>(SK_WIDE_MAX_ROWS, B - done);
+            if (!skinny_rows(bits, (h16*)outs + done * S, (const uint32_t*)matrix, (const h16*)multiplier + done * K, (const h16*)scales,
+                             (const h16*)zeros, n, K, S, g, true, (hipStream_t)stream, (const uint32_t*)sparse_mask, workspace,
+                             workspace_bytes))
+                break;
+            rc = check_launch("matvec");
+            if (rc != INT4MM_OK) return rc;
+            done += n;
+        }
+        if (done == B) return INT4MM_OK;
+    }
+    return matvec_plain(bits, (h16*)outs + done * S, matrix, (const h16*)multiplier + done * K, scales, zeros, sparse_mask, B - done, K, S, g,
+                        true, workspace, workspace_bytes, (hipStream_t)stream);
 }
 
 // One launch of the single-row kernel per batch row; `accumulate`: add onto outs (the matvec entry) or

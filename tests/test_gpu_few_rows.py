@@ -534,3 +534,15 @@ def test_two_row_blocks_of_32_on_a_narrow_output_long_k(H, bits):
     got = H.run_capi(p, d, "mtx", outs_init=np.full((1, M, S), 2.0, np.float16))
     H.assert_product_close(got, exact, f32, kind="mtx")
     assert np.array_equal(got, H.run_capi(p, d, "mtx"))
+
+
+@pytest.mark.parametrize("bits,sparse,B", [(4, False, 1100), (3, False, 1025), (4, True, 600)])
+def test_more_batch_elements_than_one_launch_takes(H, bits, sparse, B):
+    """more than 512 batch elements of one row through the matvec entry: chunks of up to 512 through the few-row kernels
+    (1 025: two chunks and the plain matvec for the last row), added onto the prior contents of outs"""
+    g = 64 if sparse else 128
+    assert "wide_rows_kernel" in H.capi.describe_launch("vec", bits, B, 1, 1024, 512, g, sparse=sparse)
+    kw = {} if bits == 4 else dict(scale_range=(0.004, 0.08), zero_const=3.5)
+    p = O.make_problem(bits=bits, K=1024, S=512, M=1, B=B, group_size=g, sparse=sparse, seed=B, **kw)
+    prior = np.random.default_rng(B).standard_normal((B, 1, 512)).astype(np.float16)
+    _check(H, p, "vec", prior=prior)

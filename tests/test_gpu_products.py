@@ -266,3 +266,22 @@ def test_matmul_five_rows_of_128_row_tiles_default_rule(H, bits, sparse):
     exact, f32 = H.oracles(p)
     got = H.run_capi(p, d, "mtx", outs_init=np.full((1, 600, 11264), 4.0, np.float16))
     H.assert_product_close(got, exact, f32, kind="mtx")
+
+
+@pytest.mark.parametrize("bits,sparse", FORMATS)
+@pytest.mark.parametrize("B,M,K,S", [(5, 130, 512, 512), (32, 20, 256, 1024), (3, 300, 320, 256), (2, 600, 1024, 384)])
+def test_batches_are_one_product_of_all_their_rows(H, bits, sparse, B, M, K, S):
+    """[B, M, K] states and [B, M, S] outputs are contiguous, so B products of M rows run as one product of B * M rows:
+    the same bits as the flattened call, and the oracle's values"""
+    capi = H.capi
+    assert capi.describe_launch("mtx", bits, B, M, K, S, 64, sparse) == capi.describe_launch("mtx", bits, 1, B * M, K, S, 64, sparse)
+    p = _problem(bits, sparse, K=K, S=S, M=M, B=B, group_size=64, seed=B + M)
+    d = H.dev_problem(p)
+    exact, f32 = H.oracles(p)
+    got = H.run_capi(p, d, "mtx", outs_init=np.full((B, M, S), 6.0, np.float16))
+    H.assert_product_close(got, exact, f32, kind=H.matmul_kind(p))
+    flat = torch.full((1, B * M, S), 6.0, dtype=torch.float16, device="cuda")
+    ws = capi.new_matmul_workspace(1, B * M, K, S, sparse)
+    capi.matmul(bits, flat, d["matrix"], d["states"].reshape(1, B * M, K), d["scales"], d["zeros"], 64, d["mask"], ws)
+    torch.cuda.synchronize()
+    assert np.array_equal(got.reshape(B * M, S), flat.cpu().numpy().reshape(B * M, S))
