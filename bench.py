@@ -49,6 +49,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-gemm", action="store_true", help="skip the M=2048 matmul leg")
+    ap.add_argument("--no-helpers", action="store_true", help="skip the pack / unpack / dequantise leg")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a 256 MiB device-to-device copy five times (a kernel of known HBM "
                          "traffic, used to scale rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
@@ -223,6 +224,36 @@ def main():
                                    "max_rel_err_vs_fp32_oracle": float(f"{err_r:.3e}")}
         result["few_rows"] = {"workload": "int4 dense, K(N)=5120 S=20480 group=128, 2, 8 and 64 rows of states "
                                           "(weights warm in the last-level cache)", **few}
+
+        # ---- the integer helpers either side of the products (pack, unpack, dequantise), HBM-bound: int4 at
+        # K = S = 16384, every array larger than the last-level cache; algorithmic bytes = inputs read + outputs written
+        if not args.no_helpers:
+            Kh = Sh = 16384
+            gen = torch.Generator(device=dev).manual_seed(5)
+            codes_sk = torch.randint(0, 16, (Sh, Kh), generator=gen, device=dev, dtype=torch.int32).to(torch.uint8)
+            keep = (torch.rand((Sh, Kh // 32, 32), generator=gen, device=dev).argsort(dim=2) < 16).to(torch.uint8).reshape(Sh, Kh)
+            m_sp = torch.zeros((Kh // 16, Sh), dtype=torch.int32, device=dev)
+            msk = torch.zeros((Kh // 32, Sh), dtype=torch.int32, device=dev)
+            codes_ks = codes_sk.t().contiguous()
+            m_de = torch.zeros((Kh // 8, Sh), dtype=torch.int32, device=dev)
+            out8 = torch.empty((Kh, Sh), dtype=torch.uint8, device=dev)
+            w16h = torch.empty((Kh, Sh), dtype=torch.float16, device=dev)
+            sch = (torch.rand((Kh // 128, Sh), generator=gen, device=dev) * 0.02).half()
+            zeh = (torch.rand((Kh // 128, Sh), generator=gen, device=dev) * 15).half()
+            n = Kh * Sh
+            legs = {"sparse_pack": (lambda: capi.sparse_pack(m_sp, msk, codes_sk, keep), 2 * n + n // 4 + n // 8),
+                    "dense_pack": (lambda: capi.dense_pack(4, m_de, codes_ks), n + n // 2),
+                    "unpack": (lambda: capi.unpack(4, out8, None, m_de, None), n // 2 + n),
+                    "dequantize": (lambda: capi.dequantize(4, w16h, m_de, sch, zeh, 128, None), n // 2 + 2 * n + 4 * (Kh // 128) * Sh),
+                    "plain_copy_same_size": (lambda: out8.copy_(codes_ks), 2 * n)}
+            helpers = {}
+            for name, (fn, nb) in legs.items():
+                us = timed(fn, warm=5, batches=5, reps=5)
+                helpers[name] = {"us": round(us, 1), "GB/s": round(nb / (us * 1e-6) / 1e9, 1),
+                                 "frac_of_hbm_peak": round(nb / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)}
+            result["helpers"] = {"workload": "int4, K(N)=S=16384 (16:32 pack: uint8 codes and mask [S, K] -> packed words and "
+                                             "mask words), cold HBM", **helpers}
+            del codes_sk, keep, codes_ks, out8, w16h
 
     # ---- CPU baseline: torch dequantise + fp32 matmul on the host (reported only)
     if not args.no_cpu:
