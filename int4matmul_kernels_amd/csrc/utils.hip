@@ -112,7 +112,8 @@ __global__ __launch_bounds__(256) void dense_pack_kernel(uint32_t* __restrict__ 
 // 16:32 packer.  Inputs are in the [S, K] orientation (row = output column): a thread takes four
 // consecutive 32-row cells of its column -- the 128 consecutive bytes of a whole cache line of each
 // input; one cell per thread left three quarters of every line to the workgroups of the next cells (180 -> 174 us
-// at K = S = 16384: what holds the kernel at 3.6 TB/s is that a wave's lines lie K bytes apart, one per lane) --
+// at K = S = 16384; staging a 64-column tile through LDS so that a wave reads whole 256-byte runs: 173 us -- it is
+// the 32-step compaction of a cell, some 250 VALU instructions, that holds the kernel at 3.7 TB/s) --
 // and writes three words per cell with lanes along the column index.
 constexpr int SPARSE_PACK_CELLS = 4;
 __global__ __launch_bounds__(256) void sparse_pack_kernel(uint32_t* __restrict__ wt_outs,
