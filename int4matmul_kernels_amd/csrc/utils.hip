@@ -64,6 +64,36 @@ __global__ __launch_bounds__(256) void unpack_kernel(uint8_t* __restrict__ codes
     }
 }
 
+// The same for four adjacent columns per thread (S a multiple of 4): a row's four codes leave as one 32-bit
+// store, a wave's store is 256 contiguous bytes of a row instead of 64 (K = S = 16384, int4: 87 -> 76 us).
+template <int BITS, bool SPARSE>
+__global__ __launch_bounds__(256) void unpack4_kernel(uint8_t* __restrict__ codes_out,
+                                                      uint8_t* __restrict__ keep_out,
+                                                      const uint32_t* __restrict__ matrix,
+                                                      const uint32_t* __restrict__ mask, int64_t K,
+                                                      int64_t S) {
+    const int64_t s = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4, blk = blockIdx.y;
+    if (s >= S) return;
+    uint32_t out[32], kept[32];
+#pragma unroll
+    for (int t = 0; t < 32; ++t) { out[t] = 0u; kept[t] = 0u; }
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        uint32_t codes[32], keep;
+        decode_block32<BITS, SPARSE>(matrix, mask, S, blk, s + c, codes, keep);
+#pragma unroll
+        for (int t = 0; t < 32; ++t) {
+            out[t] |= (codes[t] & 0xFFu) << (8 * c);
+            kept[t] |= ((keep >> t) & 1u) << (8 * c);
+        }
+    }
+#pragma unroll
+    for (int t = 0; t < 32; ++t) {
+        *reinterpret_cast<uint32_t*>(codes_out + (blk * 32 + t) * S + s) = out[t];
+        if (keep_out) *reinterpret_cast<uint32_t*>(keep_out + (blk * 32 + t) * S + s) = kept[t];
+    }
+}
+
 template <int BITS, bool SPARSE>
 __global__ __launch_bounds__(256) void dequantize_kernel(h16* __restrict__ w_out,
                                                          const uint32_t* __restrict__ matrix,
@@ -215,6 +245,14 @@ int int4mm_unpack(int bits, void* codes_out, void* keep_out, const void* matrix,
     uint8_t* k = (uint8_t*)keep_out;
     const uint32_t* m = (const uint32_t*)matrix;
     const uint32_t* msk = (const uint32_t*)sparse_mask;
+    if (out_size % 4 == 0 && (((uintptr_t)codes_out | (uintptr_t)keep_out) & 3u) == 0) {
+        const dim3 grid4((unsigned)((out_size / 4 + 255) / 256), grid.y);
+        if (msk) hipLaunchKernelGGL((unpack4_kernel<4, true>), grid4, block, 0, st, o, k, m, msk, in_size, out_size);
+        else if (bits == 4) hipLaunchKernelGGL((unpack4_kernel<4, false>), grid4, block, 0, st, o, k, m, msk, in_size, out_size);
+        else if (bits == 3) hipLaunchKernelGGL((unpack4_kernel<3, false>), grid4, block, 0, st, o, k, m, msk, in_size, out_size);
+        else hipLaunchKernelGGL((unpack4_kernel<2, false>), grid4, block, 0, st, o, k, m, msk, in_size, out_size);
+        return check_launch("unpack");
+    }
     if (msk) hipLaunchKernelGGL((unpack_kernel<4, true>), grid, block, 0, st, o, k, m, msk, in_size, out_size);
     else if (bits == 4) hipLaunchKernelGGL((unpack_kernel<4, false>), grid, block, 0, st, o, k, m, msk, in_size, out_size);
     else if (bits == 3) hipLaunchKernelGGL((unpack_kernel<3, false>), grid, block, 0, st, o, k, m, msk, in_size, out_size);
