@@ -141,10 +141,12 @@ __global__ __launch_bounds__(256) void dense_pack_kernel(uint32_t* __restrict__ 
 
 // 16:32 packer.  Inputs are in the [S, K] orientation (row = output column): a thread takes four
 // consecutive 32-row cells of its column -- the 128 consecutive bytes of a whole cache line of each
-// input; one cell per thread left three quarters of every line to the workgroups of the next cells (180 -> 174 us
-// at K = S = 16384; staging a 64-column tile through LDS so that a wave reads whole 256-byte runs: 173 us -- it is
-// the 32-step compaction of a cell, some 250 VALU instructions, that holds the kernel at 3.7 TB/s) --
-// and writes three words per cell with lanes along the column index.
+// input -- compacts the kept codes eight rows at a time (keep flags gathered by a multiply, code bytes moved to
+// the front by v_perm with selectors from a 256-entry table, squeezed to nibbles) and writes three words per cell
+// with lanes along the column index.  K = S = 16384: 180 us with one cell per thread and a 32-step loop per cell,
+// 174 with whole lines, 165 with this compaction; staging a 64-column tile through LDS so that a wave reads whole
+// 256-byte runs changed nothing (173 against 174) -- what remains is the transposition: a wave's 64 lanes read
+// lines K bytes apart.
 constexpr int SPARSE_PACK_CELLS = 4;
 __global__ __launch_bounds__(256) void sparse_pack_kernel(uint32_t* __restrict__ wt_outs,
                                                           uint32_t* __restrict__ msk_outs,
@@ -152,6 +154,20 @@ __global__ __launch_bounds__(256) void sparse_pack_kernel(uint32_t* __restrict__
                                                           const uint8_t* __restrict__ msk_in,
                                                           int64_t S, int64_t K,
                                                           int* __restrict__ bad_blocks) {
+    // compaction table: for a byte of eight keep flags, the v_perm selectors that move the kept rows' code bytes to
+    // the front in row order (0 ... 7: that row of the eight; 0x0C: a zero byte)
+    __shared__ u32x2 front[256];
+    {
+        uint32_t sel[2] = {0x0C0C0C0Cu, 0x0C0C0C0Cu};
+        int p = 0;
+        for (int r = 0; r < 8; ++r)
+            if ((threadIdx.x >> r) & 1u) {
+                sel[p >> 2] = (sel[p >> 2] & ~(0xFFu << (8 * (p & 3)))) | ((uint32_t)r << (8 * (p & 3)));
+                ++p;
+            }
+        front[threadIdx.x] = u32x2{sel[0], sel[1]};
+    }
+    __syncthreads();
     const int64_t s = (int64_t)blockIdx.x * blockDim.x + threadIdx.x, blk0 = (int64_t)blockIdx.y * SPARSE_PACK_CELLS;
     if (s >= S) return;
     const int64_t cells = K / 32;
@@ -163,6 +179,16 @@ __global__ __launch_bounds__(256) void sparse_pack_kernel(uint32_t* __restrict__
         const u32x4* mp = reinterpret_cast<const u32x4*>(msk_in + s * K + (blk0 + i) * 32);
         wq[i][0] = wp[0]; wq[i][1] = wp[1]; mq[i][0] = mp[0]; mq[i][1] = mp[1];
     }
+    // keep flags of four rows (bytes > 0) as four bits: the top bit of every non-zero byte, gathered by a multiply
+    auto flags4 = [](uint32_t m) {
+        const uint32_t nz = ((((m & 0x7F7F7F7Fu) + 0x7F7F7F7Fu) | m) & 0x80808080u) >> 7;
+        return ((nz * 0x00204081u) >> 21) & 0xFu;
+    };
+    // four code bytes (each at most 15) to four nibbles
+    auto nibbles4 = [](uint32_t o) {
+        const uint32_t n = (o | (o >> 4)) & 0x00FF00FFu;
+        return (n | (n >> 8)) & 0xFFFFu;
+    };
     int bad = 0;
 #pragma unroll
     for (int i = 0; i < SPARSE_PACK_CELLS; ++i) {
@@ -174,14 +200,15 @@ __global__ __launch_bounds__(256) void sparse_pack_kernel(uint32_t* __restrict__
         uint64_t v = 0;
         int rank = 0;
 #pragma unroll
-        for (int t = 0; t < 32; ++t) {
-            const uint32_t code = (wv[t >> 2] >> (8 * (t & 3))) & 0xFu;
-            const bool k = ((mv[t >> 2] >> (8 * (t & 3))) & 0xFFu) > 0;
-            if (k) {
-                bmsk |= 1u << t;
-                if (rank < 16) v |= (uint64_t)code << (4 * rank);
-                ++rank;
-            }
+        for (int g8 = 0; g8 < 4; ++g8) {                            // eight rows at a time
+            const uint32_t m8 = flags4(mv[2 * g8]) | (flags4(mv[2 * g8 + 1]) << 4);
+            const u32x2 sel = front[m8];
+            const uint32_t clo = wv[2 * g8] & 0x0F0F0F0Fu, chi = wv[2 * g8 + 1] & 0x0F0F0F0Fu;
+            const uint32_t kept = nibbles4(__builtin_amdgcn_perm(chi, clo, sel.x)) |
+                                  (nibbles4(__builtin_amdgcn_perm(chi, clo, sel.y)) << 16);
+            bmsk |= m8 << (8 * g8);
+            if (rank < 16) v |= (uint64_t)kept << (4 * rank);       // (codes beyond the sixteenth fall off the top)
+            rank += __builtin_popcount(m8);
         }
         msk_outs[blk * S + s] = bmsk;
         wt_outs[(2 * blk) * S + s] = (uint32_t)v;
