@@ -109,3 +109,38 @@ def test_sparse_pack_flags_wrong_popcount(H):
     assert int(bad.item()) == 1
     with pytest.raises(RuntimeError):
         H.pkg.load_extension().weight_matrix_packing(w, m, H.t(codes), H.t(keep))
+
+
+def test_sparse_pack_any_popcount_any_flag_value_high_code_bits(H):
+    """the packer is rank based (utils_kernel.cu:29-63): a row is kept when its mask byte is > 0 (any value), only the
+    low nibble of a code byte counts, the code of rank p < 16 lands at bits 4p and later ones are dropped -- checked
+    cell by cell against that closed form for blocks keeping 0 ... 32 rows; S and K / 32 not multiples of the tile"""
+    rng = np.random.default_rng(23)
+    S, K = 70, 32 * 9
+    codes = rng.integers(0, 256, (S, K), dtype=np.uint8)                       # high nibbles are noise
+    prob = rng.random((S, K // 32, 1))
+    keep = (rng.random((S, K // 32, 32)) < prob).astype(np.uint8) * rng.integers(1, 256, (S, K // 32, 32), dtype=np.uint8)
+    keep[0, 0, :] = 0
+    keep[1, 0, :] = 7
+    keep = keep.reshape(S, K)
+    w = torch.zeros((K // 16, S), dtype=torch.int32, device=H.DEV)
+    m = torch.zeros((K // 32, S), dtype=torch.int32, device=H.DEV)
+    bad = torch.zeros(1, dtype=torch.int32, device=H.DEV)
+    H.capi.sparse_pack(w, m, H.t(codes), H.t(keep), bad)
+    torch.cuda.synchronize()
+    got_w = w.cpu().numpy().view(np.uint32)
+    got_m = m.cpu().numpy().view(np.uint32)
+    wrong = 0
+    for s in range(S):
+        for b in range(K // 32):
+            bits, v, rank = 0, 0, 0
+            for t in range(32):
+                if keep[s, 32 * b + t] > 0:
+                    bits |= 1 << t
+                    if rank < 16:
+                        v |= int(codes[s, 32 * b + t] & 0xF) << (4 * rank)
+                    rank += 1
+            wrong += rank != 16
+            assert got_m[b, s] == bits, (s, b)
+            assert got_w[2 * b, s] == (v & 0xFFFFFFFF) and got_w[2 * b + 1, s] == (v >> 32), (s, b)
+    assert int(bad.item()) == wrong
