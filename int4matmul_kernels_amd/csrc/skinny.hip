@@ -973,10 +973,11 @@ static WidePlan plan_wide(int64_t R, int64_t K, int64_t S, bool sparse, int64_t 
     // (49 ... 64 rows on a narrow output: two blocks of 32 rows with half the splits instead of one block of 64 --
     // K=11008, S=4096: 28.7 -> 23.0 us; K=14336, S=4096: 31.3 -> 26.9; from 5120 columns on the single block wins on a long K)
     if (!sparse && R > 48 && R <= 64 && S <= 4096 && forced < 1) shape(32);
-    // 65 ... 512 rows of a dense format against 2048 ... 32768 columns: block height
+    // 65 ... 512 rows of a dense format against 1024 ... 32768 columns: block height
     // (up to 128, 96, 64 or 48 rows) and split by a cost model fitted to 4 900 timed launches (int4, K = 2048 ...
     // 28672, S = 4096 ... 8192, 72 ... 512 rows; its pick is within 0.3 % of the best measured candidate on average,
-    // 6.6 % at worst -- on 1 800 more launches at S = 2048 and 3072 with up to 16 splits, not used in the fit: 0.3 / 3.8 %;
+    // 6.6 % at worst -- on 1 800 more launches at S = 2048 and 3072 with up to 16 splits, not used in the fit: 0.3 / 3.8 %
+    // (and it is used from 1024 columns on: K=8192, S=1280, 104 rows 27.8 -> 21.9 us);
     // on 1 900 more at S = 11008 ... 28672, where it serves up to 192 rows: 0.3 / 10 %, the
     // rules above 6.7 / 70 %: K=2048, S=28672, 128 rows 50 -> 30 us --,
     // where the rules above were 8 % off on K <= 8192 and up to 73 % -- e.g. K=2048, S=8192, 416 rows: seven blocks
@@ -990,7 +991,7 @@ static WidePlan plan_wide(int64_t R, int64_t K, int64_t S, bool sparse, int64_t 
     struct WideCost { double per_unit[9], workgroup, split, per_way, per_tile, last_round; };
     static const WideCost dense_cost = {{0, 0, 0, 0.617, 0.707, 0, 0.912, 0, 1.059}, 3.92, -4.164, 0.798, 1.915, 3.544};
     static const WideCost sparse_cost = {{0, 0, 0, 1.12, 1.203, 0, 1.32, 0, 1.537}, 4.17, -3.744, 0.921, 1.701, 5.284};
-    if (R > 64 && S >= (sparse ? 4096 : 2048) && S <= (sparse ? 8192 : 32768) && forced < 1) {
+    if (R > 64 && S >= (sparse ? 4096 : 1024) && S <= (sparse ? 8192 : 32768) && forced < 1) {
         const WideCost& wc = sparse ? sparse_cost : dense_cost;
         const size_t room = WIDE_LDS_LIMIT - (sparse ? 4096 : 0);
         double best = 1e30;

@@ -349,7 +349,7 @@ def test_shared_staging_sparse_default_rule(H, M):
 # ---- row blocks of 96 / 128 rows (dense formats): one workgroup keeps up to eight 16-row tiles per column pair
 # and stages two rows of states per thread.  Taken where K is not split at all or split into long shares.
 @pytest.mark.parametrize("bits", [4, 3, 2])
-@pytest.mark.parametrize("M,K,S,g", [(100, 512, 512, 64), (128, 512, 256, 128), (70, 320, 1024, 64), (65, 448, 256, -1),
+@pytest.mark.parametrize("M,K,S,g", [(100, 512, 512, 64), (128, 512, 256, 128), (70, 320, 768, 64), (65, 448, 256, -1),
                                      (256, 512, 512, 128), (129, 512, 256, 64), (200, 256, 768, 64)])
 def test_tall_row_blocks(H, bits, M, K, S, g):
     tiles = H.capi.describe_launch("mtx", bits, 1, M, K, S, g)
