@@ -199,13 +199,21 @@ def main():
         with torch.cuda.stream(stream):
             lib_us = timed(lambda: torch.matmul(xs[0], w16_dev))
         del w16_dev
+        # the shader clock the power management leaves this kernel (rocm-smi sampled every 0.1 s while it is
+        # launched back to back for two seconds): the 2.5 PFLOP/s peak assumes 2.4 GHz on all 256 compute units
+        from int4matmul_kernels_amd.harness import shader_clock_under_load
+        sclk = shader_clock_under_load(lambda: capi.matmul(4, om, m, xs, sc, ze, g, None, ws_mm), 2.0)
+        peak_at_clock = MFMA_FP16_PEAK_TFLOPS * sclk / 2400.0 if sclk else None
         result["gemm"] = {"workload": "int4 dense matmul M=2048 K(N)=5120 S=20480 group=128",
                           "vendor_fp16_gemm_same_shape": {"us": round(lib_us, 2),
                                                           "tflops": round(flops / (lib_us * 1e-6) / 1e12, 1)},
                           "us": round(mm_us, 2), "tflops": round(tf, 1),
                           "roofline": {"bound": "mfma", "achieved": round(tf, 1), "peak": MFMA_FP16_PEAK_TFLOPS,
                                        "unit": "TFLOP/s", "frac": round(tf / MFMA_FP16_PEAK_TFLOPS, 4),
-                                       "traffic": MATMUL_TRAFFIC_BYTES},
+                                       "traffic": MATMUL_TRAFFIC_BYTES,
+                                       "sclk_mhz_under_load": sclk,
+                                       "peak_at_clock": round(peak_at_clock, 1) if peak_at_clock else None,
+                                       "frac_at_clock": round(tf / peak_at_clock, 4) if peak_at_clock else None},
                           "max_rel_err_vs_fp32_oracle": float(f"{mm_err:.3e}")}
 
         # ---- the few-row products in between (a batch of decoding requests): 2, 8 and 64 rows, same weights

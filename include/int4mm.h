@@ -91,8 +91,7 @@ INT4MM_API int int4mm_abi_version(void);
  * shape allows a split at all), 7 = 1: the tiles of a matmul's last, partly
  * filled round are not split, 8 = the few-row kernel whose waves share the
  * staged states: 1 = never, n >= 2 = from n rows on whatever the shape,
- * 9 = address of a device buffer of int64 [workgroups][8][16]: the dense int4 matvec then runs
- * its instrumented variant and records time stamps there (see matvec_timeline.py),
+ * 9 = unused,
  * 10 = polls after which a matvec hand-over gives up (failure-handling tests). */
 INT4MM_API int int4mm_tune(int key, int64_t value);
 
@@ -102,11 +101,12 @@ INT4MM_API int int4mm_tune(int key, int64_t value);
  *   dense : R * 32 == K * bits         sparse (bits == 4) : R * 16 == K
  *   K % 64 == 0, S % 64 == 0 (README.md:9), B, M >= 1 (B*M*S == 0 returns OK)
  *   group_size < 0 (one group) or group_size % 64 == 0; g * G >= K
- * Two limits the reference does not have:
- *   int4mm_matvec: K <= 458752 (INT4MM_ERR_SHAPE beyond: a workgroup stages the states
- *   of its K range in 64 KB of LDS, 224 units of 64 rows, and K is cut at most 32 ways);
- *   int4mm_matvec needs a workspace of int4mm_workspace_bytes(S) bytes even for shapes it
- *   would not split (INT4MM_ERR_WORKSPACE without one; it does not fall back).
+ * One requirement the reference does not have:
+ *   int4mm_matvec needs a workspace of int4mm_workspace_bytes(S) bytes, whatever launch
+ *   shape the product takes (INT4MM_ERR_WORKSPACE without one; it does not fall back).
+ * (A K beyond 458752 -- what one launch covers: 32 ranges of 224 units of 64 rows -- runs as
+ * several launches, each adding onto the result of the one before.  The only shape refused
+ * for its length is a single quantisation group longer than that on a still longer K.)
  */
 typedef struct int4mm_shape {
     int64_t batch;        /* B */
@@ -127,6 +127,9 @@ typedef struct int4mm_shape {
  * kept zero -- hand-over slots, arrival counters -- and the upper half is scratch
  * for partial tiles), so always pass the size the buffer was zero-filled with. */
 INT4MM_API size_t int4mm_workspace_bytes(int64_t max_out_size);
+/* Zero-fills a workspace with a kernel on `stream` (no allocation, no memset node: it may be
+ * recorded into a graph).  workspace == NULL with workspace_bytes == 0 means the array built
+ * into the library that int4mm_matvec_static works on. */
 INT4MM_API int int4mm_workspace_init(void* workspace, size_t workspace_bytes, void* stream);
 
 /* Health of a workspace.  The matvec's workgroups hand partial sums over through the workspace;
@@ -134,7 +137,9 @@ INT4MM_API int int4mm_workspace_init(void* workspace, size_t workspace_bytes, vo
  * that wait ever runs out (it cannot while the GPU dispatches workgroups in order), the affected
  * outputs are NaN, the workspace is marked, and every later matvec on it returns NaN too -- never a
  * silently wrong number -- until int4mm_workspace_init has zero-filled it again.  This call copies
- * the mark back on `stream`, waits for it and returns INT4MM_ERR_HANDOVER if it is set.  No
+ * the mark back on `stream`, waits for it and returns INT4MM_ERR_HANDOVER if it is set.
+ * workspace == NULL with workspace_bytes == 0 asks about the array built into the library
+ * (int4mm_matvec_static), which int4mm_workspace_init(NULL, 0, stream) zero-fills again.  No
  * counterpart in the reference, whose atomics cannot time out (matvec_kernel.cu:263). */
 INT4MM_API int int4mm_workspace_status(void* workspace, size_t workspace_bytes, void* stream);
 
@@ -168,13 +173,19 @@ INT4MM_API int int4mm_matvec(int bits, void* outs, const void* matrix, const voi
 
 /* int4mm_matvec for callers that cannot allocate device memory (code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc): same arguments without
- * the workspace, same kernels, same results bit for bit.  The hand-over slots and split-K
- * partials live in a 16.8 MB device array built into the library (each GPU the library
+ * the workspace, same kernels.  Results are bit for bit those of int4mm_matvec on a workspace
+ * that allows the same launch plan: always for one row of states; for several batch entries
+ * when that workspace has int4mm_matmul_workspace_bytes() and the few-row kernels' partial
+ * sums fit the array's scratch half (8.4 MB) -- a smaller workspace, or larger partials, makes
+ * one of the two run unsplit, which changes the summation order, not the accuracy class.  The
+ * hand-over slots and split-K partials live in a 16.8 MB device array built into the library (each GPU the library
  * runs on holds its copy until the process ends), which covers out_size <= 32768; a wider
  * product returns INT4MM_ERR_WORKSPACE.  The call allocates and frees nothing.  Its first
  * call on a device looks up that device's copy of the array (make it once outside any
  * graph capture).  All calls on one GPU share the array: calls that overlap in time on one
  * GPU (two streams) race, exactly as two int4mm_matvec calls sharing one workspace would.
+ * A hand-over that times out marks the array like any workspace: int4mm_workspace_status(NULL,
+ * 0, stream) reports it and int4mm_workspace_init(NULL, 0, stream) clears it.
  * No counterpart in the reference, whose matvec allocates an fp32 temporary per call
  * (matvec_kernel.cu:351). */
 INT4MM_API int int4mm_matvec_static(int bits, void* outs, const void* matrix, const void* multiplier,

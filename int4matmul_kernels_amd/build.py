@@ -56,17 +56,6 @@ def build_hip_library(verbose: bool = False) -> str:
     return LIB
 
 
-PROBE = os.path.join(PKG, "read_probe")
-
-
-def build_read_probe() -> str:
-    """Stand-alone diagnostic (csrc/read_probe.hip): the read-only floor of a matvec."""
-    _run([HIPCC, "-O3", "-std=c++17", f"--offload-arch={ARCH}", "-Xclang", "-target-feature", "-Xclang",
-          "-packed-fp32-ops", "-Wno-unused-result", "-Wno-unknown-warning-option", "-Wno-unused-command-line-argument",
-          os.path.join(CSRC, "read_probe.hip"), "-o", PROBE])
-    return PROBE
-
-
 def extension_path() -> str:
     return os.path.join(PKG, "int4matmul" + sysconfig.get_config_var("EXT_SUFFIX"))
 
@@ -99,7 +88,6 @@ def build_extension(verbose: bool = False) -> str:
 def build_all(verbose: bool = False):
     lib = build_hip_library(verbose)
     ext = build_extension(verbose)
-    build_read_probe()
     return lib, ext
 
 

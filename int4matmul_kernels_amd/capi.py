@@ -111,9 +111,17 @@ def describe_launch(product, bits, batch, seq_len, in_size, out_size, group_size
     return buf.value.decode()
 
 
-def workspace_status(workspace):
-    """0 if healthy; raises Int4mmError(code 9) after a matvec hand-over timed out on it"""
-    _check(lib().int4mm_workspace_status(_ptr(workspace), workspace.numel(), _stream()), "int4mm_workspace_status")
+def workspace_status(workspace=None):
+    """0 if healthy; raises Int4mmError(code 9) after a matvec hand-over timed out on it
+    (``None``: the array built into the library that ``matvec_static`` works on)"""
+    n = 0 if workspace is None else workspace.numel()
+    _check(lib().int4mm_workspace_status(_ptr(workspace), n, _stream()), "int4mm_workspace_status")
+
+
+def workspace_init(workspace=None):
+    """zero-fill a workspace with a kernel on the current stream (``None``: the built-in array)"""
+    n = 0 if workspace is None else workspace.numel()
+    _check(lib().int4mm_workspace_init(_ptr(workspace), n, _stream()), "int4mm_workspace_init")
 
 
 def new_workspace(out_size: int, device="cuda"):

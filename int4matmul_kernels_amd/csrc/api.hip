@@ -111,7 +111,7 @@ int int4mm_abi_version(void) { return 1; }
 // 6 = matmul split-K factor (1 = never, 2..8 = forced where the shape allows a split),
 // 7 = 1: the tiles of a matmul's last, partly filled round are not split,
 // 8 = 1: 33 .. 96 rows take the few-row kernel whose waves stage their own states,
-// 9 = address of the matvec's time-stamp buffer, 10 = polls before a matvec hand-over gives up.
+// 9 = unused, 10 = polls before a matvec hand-over gives up.
 int int4mm_tune(int key, int64_t value) {
     if (key < 0 || key >= TUNE_COUNT) return INT4MM_ERR_SHAPE;
     g_tuning[key] = value;
@@ -123,8 +123,13 @@ size_t int4mm_workspace_bytes(int64_t max_out_size) {
     return 2 * (matvec_slots_bytes(max_out_size) + 4096);
 }
 
+// workspace == NULL: the array built into the library (what int4mm_matvec_static works on); a fill kernel on
+// `stream`, no allocation, no memset node
 int int4mm_workspace_init(void* workspace, size_t workspace_bytes, void* stream) {
-    if (workspace == nullptr) return INT4MM_ERR_NULL;
+    if (workspace == nullptr) {
+        if (workspace_bytes != 0) return INT4MM_ERR_NULL;
+        if (!static_scratch(&workspace, &workspace_bytes)) return INT4MM_ERR_LAUNCH;
+    }
     if (workspace_bytes < 4096) return INT4MM_ERR_WORKSPACE;
     size_t n = workspace_bytes / 4;
     hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
@@ -152,7 +157,10 @@ int int4mm_describe_launch(int product, int bits, const int4mm_shape* shape, int
 // back on `stream` and waits for it.)  After INT4MM_ERR_HANDOVER every matvec on the workspace returns
 // NaN until int4mm_workspace_init has run again.
 int int4mm_workspace_status(void* workspace, size_t workspace_bytes, void* stream) {
-    if (workspace == nullptr) return INT4MM_ERR_NULL;
+    if (workspace == nullptr) {                                  // the built-in array of int4mm_matvec_static
+        if (workspace_bytes != 0) return INT4MM_ERR_NULL;
+        if (!static_scratch(&workspace, &workspace_bytes)) return INT4MM_ERR_LAUNCH;
+    }
     const WorkspaceParts p = workspace_parts(workspace, workspace_bytes);
     if (p.counters == nullptr) return INT4MM_ERR_WORKSPACE;
     uint32_t word = 0;

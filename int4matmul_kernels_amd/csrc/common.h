@@ -55,6 +55,16 @@ __device__ __forceinline__ float wave_sum(float v) {
     return (r0 + r1) + (r2 + r3);
 }
 
+// (w & mask) | magic is one VALU op (v_and_or_b32) only when both constants sit in registers: a VOP3
+// instruction of this ISA cannot carry two literals.  Such constants are materialised once through an
+// opaque move, and the expression itself is left to the compiler (so that it also tracks the VALU -> MFMA
+// operand hazards, which it cannot do through inline assembly).
+__device__ __forceinline__ uint32_t in_vgpr(uint32_t literal) {
+    uint32_t r;
+    asm("v_mov_b32 %0, %1" : "=v"(r) : "s"(literal));
+    return r;
+}
+
 // ---- one code -> fp16 weight, the two roundings of the linear mode and the
 // single-rounded fused multiply-add of the exponent mode.
 template <int BITS>
@@ -106,7 +116,7 @@ int validate_product(int bits, const void* outs, const void* matrix, const void*
                      const int4mm_shape* sh, bool matvec);
 int64_t tuning(int key);                       // see int4mm_tune (values are per host thread)
 enum TuneKey { TUNE_MV_WAVES = 0, TUNE_MV_UNITS = 1, TUNE_MV_LK = 2, TUNE_MM_VARIANT = 3, TUNE_MV_NOPF = 4,
-               TUNE_NO_SKINNY = 5, TUNE_MM_SPLIT = 6, TUNE_MM_TAIL = 7, TUNE_NO_WIDE = 8, TUNE_MV_TIMELINE = 9,
+               TUNE_NO_SKINNY = 5, TUNE_MM_SPLIT = 6, TUNE_MM_TAIL = 7, TUNE_NO_WIDE = 8, TUNE_RESERVED_9 = 9,
                TUNE_MV_SPIN = 10, TUNE_COUNT = 11 };
 
 // int4mm_describe_launch: while this thread is "noting", a launcher records the kernel and launch
@@ -157,6 +167,9 @@ inline size_t matvec_slots_bytes(int64_t out_size) {
     if (out_size < 0) out_size = 0;
     return 4096 + (size_t)((out_size + 255) / 256 * 256) * 8 * 32;
 }
+// the array built into the library that int4mm_matvec_static uses as its workspace (csrc/matvec.hip): the
+// current device's copy and its size; false if the runtime cannot resolve it
+bool static_scratch(void** ptr, size_t* bytes);
 inline size_t round_to_page(size_t n) { return (n + 4095) & ~size_t(4095); }
 
 }  // namespace i4

@@ -115,17 +115,10 @@ __device__ __forceinline__ void dequant_cell_generic(const Cell<BITS, SPARSE>& c
 // halves of a register, so that mask-and-OR yields the half2 {1024 + q_even,
 // 64 + q_odd}; subtracting {1024, 64} is exact, then the reference's own two
 // roundings follow: fp16(q - z), fp16(. * s).
-// mask / magic constants held in VGPRs so that v_and_or_b32 is selected (a VOP3
-// encoding cannot carry two different literals); the expression stays visible to
-// the compiler, which has to track the VALU -> MFMA operand hazards
-__device__ __forceinline__ uint32_t vgpr_const(uint32_t literal) {
-    uint32_t r;
-    asm("v_mov_b32 %0, %1" : "=v"(r) : "s"(literal));
-    return r;
-}
+// (mask / magic constants are held in registers, in_vgpr, so that v_and_or_b32 is selected)
 
 __device__ __forceinline__ h16x8 dequant_word_int4(uint32_t u, h16x2 negz, h16x2 s2) {
-    const uint32_t MSK = vgpr_const(0x00F0000Fu), MAGIC = vgpr_const(0x54006400u);
+    const uint32_t MSK = in_vgpr(0x00F0000Fu), MAGIC = in_vgpr(0x54006400u);
     const h16x2 unmagic = {(h16)-1024.0f, (h16)-64.0f};
     const uint32_t lo = __builtin_amdgcn_perm(u, u, 0x01000100u);    // bytes B0 B1 B0 B1
     const uint32_t hi = __builtin_amdgcn_perm(u, u, 0x03020302u);    // bytes B2 B3 B2 B3
@@ -351,7 +344,7 @@ __device__ __forceinline__ h16x8 dequant_chunk_mixed(uint32_t bits, bool expo, h
     uint32_t h[4];
     h16x2 unmagic;
     if constexpr (BITS == 4) {
-        const uint32_t MSK = vgpr_const(0x00F0000Fu), MAGIC = vgpr_const(0x54006400u);
+        const uint32_t MSK = in_vgpr(0x00F0000Fu), MAGIC = in_vgpr(0x54006400u);
         unmagic = h16x2{(h16)-1024.0f, (h16)-64.0f};
         const uint32_t lo = __builtin_amdgcn_perm(bits, bits, 0x01000100u);
         const uint32_t hi = __builtin_amdgcn_perm(bits, bits, 0x03020302u);

@@ -55,7 +55,6 @@ struct MatvecArgs {
     int splits;             // == gridDim.y
     uint32_t* sticky;       // hand-over error word of the workspace (non-zero: poisoned)
     int spin_limit;         // polls before a reader gives up
-    uint64_t* timeline;     // instrumented variant only: 16 time stamps per wave (8 wave slots per workgroup)
     int rows;               // several rows of states in one pass (NR = 4 kernels): how many (2 .. 4), K apart in x, S apart in outs
     int accumulate;         // ... and whether they add onto outs (the matvec entry) or overwrite it (the matmul entry)
 };
@@ -95,16 +94,7 @@ __device__ __forceinline__ void load_unit(Unit<BITS, SPARSE>& u, const MatvecArg
     }
 }
 
-// (w & mask) | magic is one VALU op (v_and_or_b32) only when both constants sit
-// in registers: a VOP3 instruction of this ISA cannot carry two literals.  The
-// constants are therefore materialised once through an opaque move, and the
-// expression itself is left to the compiler (so that it also tracks the
-// VALU -> MFMA operand hazards, which it cannot do through inline assembly).
-__device__ __forceinline__ uint32_t in_vgpr(uint32_t literal) {
-    uint32_t r;
-    asm("v_mov_b32 %0, %1" : "=v"(r) : "s"(literal));
-    return r;
-}
+// (mask and magic are held in registers, in_vgpr: one v_and_or_b32)
 __device__ __forceinline__ uint32_t and_or(uint32_t w, uint32_t mask, uint32_t magic) {
     return (w & mask) | magic;
 }
@@ -398,11 +388,6 @@ __device__ __forceinline__ uint64_t slot_load(const uint64_t* p) {
 // (more registers); without it a lane group loads and processes one unit at a
 // time and relies on the other resident waves to cover the latency.
 //
-// TL: instrumented variant (dense int4 only) that records, per wave, the 100 MHz wall clock at
-// entry (0), after its first requests (1), after the staging barrier (2), after each of its first
-// nine units (3..11), after the workgroup's reduction (12) and at the end (13), and the hardware
-// ids of where it ran (15).
-//
 // NR = 2, 4: up to two / four rows of states in one pass over the weights (dense formats).  The 4x4x4 MFMA
 // computes a 4 x 4 block per four lanes; with one row of states every lane passes the same four
 // states as its row of A and three of the four result registers repeat the first.  Here lane
@@ -410,11 +395,11 @@ __device__ __forceinline__ uint64_t slot_load(const uint64_t* p) {
 // column: the same instructions and the same weight traffic give four rows of outputs (NR = 2:
 // lanes 4b + i and 4b + i + 2 pass row i, two registers are used).  Staged states, unit sums, the
 // reduction area and the hand-over slots (slot row = split * NR + row) are kept per row.
-template <int BITS, bool SPARSE, int LK, bool PF, bool TL = false, int NR = 1>
+template <int BITS, bool SPARSE, int LK, bool PF, int NR = 1>
 __global__ __launch_bounds__(MV_MAX_WAVES * WAVE)
 void matvec_kernel(MatvecArgs a) {
     constexpr bool FAST = Fmt<BITS, SPARSE>::FAST;
-    static_assert(NR == 1 || ((NR == 2 || NR == 4) && FAST && !SPARSE && !TL), "several rows: dense formats only");
+    static_assert(NR == 1 || ((NR == 2 || NR == 4) && FAST && !SPARSE), "several rows: dense formats only");
     constexpr int LC = WAVE / LK;                 // column lanes per lane group
     constexpr int COLS = LC * 4;                  // columns per strip
 
@@ -431,17 +416,6 @@ void matvec_kernel(MatvecArgs a) {
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6, nwaves = blockDim.x >> 6;
     const int cl = lane % LC, kl = lane / LC;
     const int strip = blockIdx.x, split = blockIdx.y;
-    int stamped_units = 0;
-    auto stamp = [&](int k) {
-        if constexpr (TL) {
-            __builtin_amdgcn_sched_barrier(0);
-            uint64_t c = wall_clock64();
-            if (k == 15) c = ((uint64_t)__builtin_amdgcn_s_getreg((31 << 11) | 20) << 32) | __builtin_amdgcn_s_getreg((31 << 11) | 4);
-            if (lane == 0) a.timeline[((int64_t)(blockIdx.y * gridDim.x + blockIdx.x) * MV_MAX_WAVES + wave) * 16 + k] = c;
-            __builtin_amdgcn_sched_barrier(0);
-        }
-    };
-    stamp(0);
     const int col = strip * COLS + cl * 4;
     const bool col_ok = col < a.S;
 
@@ -489,7 +463,6 @@ void matvec_kernel(MatvecArgs a) {
     if constexpr (PF) {
         if (work_b) load_unit(ub, a, u + ng, col);
     }
-    stamp(1);
 
     if constexpr (SPARSE) {
         // selector table: for mask byte b, pair j = (row j, row j+4): byte 0 picks the code of
@@ -594,7 +567,6 @@ void matvec_kernel(MatvecArgs a) {
         }
         __syncthreads();
     }
-    stamp(2);
 
     float y[4] = {0.f, 0.f, 0.f, 0.f};
     float yr[NR == 1 ? 1 : 4][NR == 1 ? 1 : NR] = {};       // NR rows: yr[column][row] instead of y
@@ -663,13 +635,11 @@ void matvec_kernel(MatvecArgs a) {
             bool has_b = work_b;
             for (;;) {
                 finish_unit(ua, u);
-                if (stamped_units < 9) stamp(3 + stamped_units++);
                 if (!has_b) break;
                 const int u2 = u + 2 * ng, u3 = u + 3 * ng;
                 const bool has_a = u2 < wg_u1;
                 if (has_a) load_unit(ua, a, u2, col);
                 finish_unit(ub, u + ng);
-                if (stamped_units < 9) stamp(3 + stamped_units++);
                 if (!has_a) break;
                 has_b = u3 < wg_u1;
                 if (has_b) load_unit(ub, a, u3, col);
@@ -678,7 +648,6 @@ void matvec_kernel(MatvecArgs a) {
         } else {
             for (;;) {
                 finish_unit(ua, u);
-                if (stamped_units < 9) stamp(3 + stamped_units++);
                 u += ng;
                 if (u >= wg_u1) break;
                 load_unit(ua, a, u, col);
@@ -801,7 +770,6 @@ void matvec_kernel(MatvecArgs a) {
                 for (int k = 0; k < LK; ++k) total[i] += red[(w * 64 + k * LC) * 4 + j];
         }
     }
-    stamp(12);
     auto for_owned = [&](auto&& fn) {
 #pragma unroll
         for (int i = 0; i < MAXC; ++i) {
@@ -812,7 +780,6 @@ void matvec_kernel(MatvecArgs a) {
     };
     if (a.splits == 1) {
         for_owned([&](int i, int ocol) { a.outs[ocol] = (h16)((a.accumulate ? (float)a.outs[ocol] : 0.f) + total[i]); });
-        stamp(13); stamp(15);
         return;
     }
 
@@ -823,7 +790,6 @@ void matvec_kernel(MatvecArgs a) {
     // next call and writes the result.
     if (split != a.splits - 1) {
         for_owned([&](int i, int ocol) { slot_store(&a.slots[(int64_t)split * a.S + ocol], total[i], SLOT_FULL); });
-        stamp(13); stamp(15);
         return;
     }
     // (a hand-over that timed out earlier may have left late slots behind: the workspace stays
@@ -861,7 +827,6 @@ void matvec_kernel(MatvecArgs a) {
         if (!ok) __hip_atomic_store(a.sticky, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         a.outs[ocol] = ok ? (h16)sum : (h16)__builtin_nanf("");
     });
-    stamp(13); stamp(15);
 }
 
 // LDS of a launch: staged states + per-unit sums (per row), or the reduction area (4 floats per thread and row)
@@ -874,7 +839,7 @@ static size_t matvec_lds_bytes(int units_per_wg, int threads, int nr) {
 template <int BITS, int NR>
 static void launch_rows(const MatvecArgs& a, int lk, bool pf, dim3 grid, dim3 block, hipStream_t st) {
     const size_t lds = matvec_lds_bytes<BITS, false>(a.units_per_wg, (int)block.x, NR);
-#define I4_LAUNCH(LK_, PF_) hipLaunchKernelGGL((matvec_kernel<BITS, false, LK_, PF_, false, NR>), grid, block, lds, st, a)
+#define I4_LAUNCH(LK_, PF_) hipLaunchKernelGGL((matvec_kernel<BITS, false, LK_, PF_, NR>), grid, block, lds, st, a)
     if (lk == 1) { if (pf) I4_LAUNCH(1, true); else I4_LAUNCH(1, false); }
     else if (lk == 2) { if (pf) I4_LAUNCH(2, true); else I4_LAUNCH(2, false); }
     else { if (pf) I4_LAUNCH(4, true); else I4_LAUNCH(4, false); }
@@ -884,12 +849,7 @@ static void launch_rows(const MatvecArgs& a, int lk, bool pf, dim3 grid, dim3 bl
 template <int BITS, bool SPARSE>
 static void launch(const MatvecArgs& a, int lk, bool pf, dim3 grid, dim3 block, hipStream_t st) {
     const size_t lds = matvec_lds_bytes<BITS, SPARSE>(a.units_per_wg, (int)block.x, 1);
-#define I4_LAUNCH(LK_, PF_) do { \
-        if constexpr (BITS == 4 && !SPARSE) { \
-            if (a.timeline) { hipLaunchKernelGGL((matvec_kernel<BITS, SPARSE, LK_, PF_, true>), grid, block, lds, st, a); break; } \
-        } \
-        hipLaunchKernelGGL((matvec_kernel<BITS, SPARSE, LK_, PF_, false>), grid, block, lds, st, a); \
-    } while (0)
+#define I4_LAUNCH(LK_, PF_) hipLaunchKernelGGL((matvec_kernel<BITS, SPARSE, LK_, PF_>), grid, block, lds, st, a)
     if (lk == 1) { if (pf) I4_LAUNCH(1, true); else I4_LAUNCH(1, false); }
     else if (lk == 2) { if (pf) I4_LAUNCH(2, true); else I4_LAUNCH(2, false); }
     else { if (pf) I4_LAUNCH(4, true); else I4_LAUNCH(4, false); }
@@ -964,7 +924,7 @@ static MatvecShape plan_matvec(int64_t S, int units_total) {
 bool i4::matvec_rows(int bits, h16* outs, const uint32_t* matrix, const h16* x, const h16* scales, const h16* zeros,
                      int64_t R, int64_t K, int64_t S, int64_t group_size, bool accumulate, hipStream_t st,
                      void* workspace, size_t workspace_bytes) {
-    if (R < 2 || R > 4 || K % 64 != 0 || S % 4 != 0 || tuning(TUNE_MV_TIMELINE)) return false;
+    if (R < 2 || R > 4 || K % 64 != 0 || S % 4 != 0) return false;
     // measured against the few-row kernel (S = 11008 ... 32768, warm weights): 10 - 26 % faster up to K = 5120
     // (K=5120, S=20480: 2 / 3 / 4 rows 14.0 / 15.4 / 17.1 against 18.4 / 18.1 / 18.3 us; K=4096, S=11008: 9.5 / 11.1 /
     // 12.3 against 11.3 / 12.5 / 12.4), 3 - 14 % slower from K = 6144 on, where staging four rows of states per
@@ -1002,7 +962,6 @@ bool i4::matvec_rows(int bits, h16* outs, const uint32_t* matrix, const h16* x, 
     a.units_per_wg = ms.upwg;
     a.group_units = (int)(group_size / 64 > 0x7FFFFFF ? 0x7FFFFFF : group_size / 64);
     a.splits = ms.splits;
-    a.timeline = nullptr;
     a.sticky = ms.splits > 1 ? reinterpret_cast<uint32_t*>(ws.counters - 8) : nullptr;
     a.spin_limit = tuning(TUNE_MV_SPIN) > 0 ? (int)tuning(TUNE_MV_SPIN) : MV_SPIN_LIMIT;
     a.rows = (int)R;
@@ -1033,7 +992,8 @@ static int matvec_plain(int bits, void* outs, const void* matrix, const void* mu
 bool i4::matvec_one_row(int bits, h16* outs, const uint32_t* matrix, const uint32_t* sparse_mask, const h16* x, const h16* scales,
                         const h16* zeros, int64_t K, int64_t S, int64_t group_size, hipStream_t st, void* workspace,
                         size_t workspace_bytes, int* rc) {
-    if (K % 64 != 0 || S % 4 != 0 || tuning(TUNE_MV_TIMELINE)) return false;
+    if (K % 64 != 0 || S % 4 != 0) return false;
+    if (K / 64 > (int64_t)MV_MAX_SPLITS * MV_MAX_UNITS_WG) return false;        // (several launches: the tile kernels take it)
     const MatvecShape ms = plan_matvec(S, (int)(K / 64));
     if (ms.upwg > MV_MAX_UNITS_WG) return false;
     if (ms.splits > 1 && workspace_parts(workspace, workspace_bytes).slots_bytes < matvec_slots_bytes(S)) return false;
@@ -1049,8 +1009,9 @@ static int matvec_impl(int bits, void* outs, const void* matrix, const void* mul
     if (rc != INT4MM_OK) return rc;
     const int64_t B = shape->batch, K = shape->in_size, S = shape->out_size;
     if (B * shape->seq_len * S == 0) return INT4MM_OK;
+    // the documented rule, whichever launch shape the product takes: a workspace of int4mm_workspace_bytes(S)
+    if (workspace_parts(workspace, workspace_bytes).slots_bytes < matvec_slots_bytes(S)) return INT4MM_ERR_WORKSPACE;
 
-    const int units_total = (int)(K / 64);
     const int64_t g = shape->group_size < 0 ? ONE_GROUP : shape->group_size;
 
     // several batch elements of one row each: one pass over the weights for all of them
@@ -1085,51 +1046,62 @@ static int matvec_impl(int bits, void* outs, const void* matrix, const void* mul
 }
 
 // One launch of the single-row kernel per batch row; `accumulate`: add onto outs (the matvec entry) or
-// overwrite it (a single row through the matmul entry).
+// overwrite it (a single row through the matmul entry).  A launch stages its share of the states in LDS and
+// cuts K at most MV_MAX_SPLITS ways, so it covers MV_MAX_SPLITS x MV_MAX_UNITS_WG units of K; a longer K (the
+// reference's grid covers any: matvec_kernel.cu:339-347) goes in ranges of that many units, each a whole
+// number of quantisation groups, the later ones adding onto the result of the earlier.
 static int matvec_plain(int bits, void* outs, const void* matrix, const void* multiplier, const void* scales, const void* zeros,
                         const void* sparse_mask, int64_t B, int64_t K, int64_t S, int64_t g, bool accumulate, void* workspace,
                         size_t workspace_bytes, hipStream_t st) {
-    const int units_total = (int)(K / 64);
-    const MatvecShape ms = plan_matvec(S, units_total);
-    const int lk = ms.lk, waves = ms.waves, upwg = ms.upwg, splits = ms.splits, strips = ms.strips;
-    if (upwg > MV_MAX_UNITS_WG) return INT4MM_ERR_SHAPE;
-    if (splits > 1 && workspace_parts(workspace, workspace_bytes).slots_bytes < matvec_slots_bytes(S))
-        return INT4MM_ERR_WORKSPACE;
-    // software prefetch only pays when lane groups walk several units
-    const bool pf = upwg >= 3 * waves * lk && tuning(TUNE_MV_NOPF) == 0;
+    const int64_t units_all = K / 64;
+    const int64_t gu = g / 64 > 0x7FFFFFF ? 0x7FFFFFF : g / 64;               // units per quantisation group
+    int64_t range_units = (int64_t)MV_MAX_SPLITS * MV_MAX_UNITS_WG;
+    if (units_all > range_units) {
+        if (gu > range_units && gu < units_all) return INT4MM_ERR_SHAPE;        // (a group longer than a launch covers)
+        if (gu <= range_units) range_units = range_units / gu * gu;
+    }
+    for (int64_t u0 = 0; u0 < units_all; u0 += range_units) {
+        const int units_total = (int)std::min(range_units, units_all - u0);
+        const MatvecShape ms = plan_matvec(S, units_total);
+        const int lk = ms.lk, waves = ms.waves, upwg = ms.upwg, splits = ms.splits, strips = ms.strips;
+        if (upwg > MV_MAX_UNITS_WG) return INT4MM_ERR_SHAPE;
+        if (splits > 1 && workspace_parts(workspace, workspace_bytes).slots_bytes < matvec_slots_bytes(S))
+            return INT4MM_ERR_WORKSPACE;
+        // software prefetch only pays when lane groups walk several units
+        const bool pf = upwg >= 3 * waves * lk && tuning(TUNE_MV_NOPF) == 0;
 
-    MatvecArgs a;
-    a.matrix = (const uint32_t*)matrix;
-    a.mask = (const uint32_t*)sparse_mask;
-    a.scales = (const h16*)scales;
-    a.zeros = (const h16*)zeros;
-    a.slots = (uint64_t*)workspace;
-    a.K = (int)K;
-    a.S = (int)S;
-    a.units_total = units_total;
-    a.units_per_wg = upwg;
-    a.group_units = (int)(g / 64 > 0x7FFFFFF ? 0x7FFFFFF : g / 64);
-    a.splits = splits;
-    a.timeline = (uint64_t*)(uintptr_t)tuning(TUNE_MV_TIMELINE);
-    a.sticky = splits > 1 ? reinterpret_cast<uint32_t*>(workspace_parts(workspace, workspace_bytes).counters - 8) : nullptr;
-    a.spin_limit = tuning(TUNE_MV_SPIN) > 0 ? (int)tuning(TUNE_MV_SPIN) : MV_SPIN_LIMIT;
-    a.rows = 1;
-    a.accumulate = accumulate ? 1 : 0;
+        MatvecArgs a;
+        // the range's first packed row, mask row and group row (u0 is a multiple of the group size, or 0)
+        a.matrix = (const uint32_t*)matrix + (sparse_mask ? u0 * 4 : u0 * 2 * bits) * S;
+        a.mask = sparse_mask ? (const uint32_t*)sparse_mask + u0 * 2 * S : nullptr;
+        a.scales = (const h16*)scales + (u0 / gu) * S;
+        a.zeros = (const h16*)zeros + (u0 / gu) * S;
+        a.slots = (uint64_t*)workspace;
+        a.K = units_total * 64;
+        a.S = (int)S;
+        a.units_total = units_total;
+        a.units_per_wg = upwg;
+        a.group_units = (int)gu;
+        a.splits = splits;
+        a.sticky = splits > 1 ? reinterpret_cast<uint32_t*>(workspace_parts(workspace, workspace_bytes).counters - 8) : nullptr;
+        a.spin_limit = tuning(TUNE_MV_SPIN) > 0 ? (int)tuning(TUNE_MV_SPIN) : MV_SPIN_LIMIT;
+        a.rows = 1;
+        a.accumulate = (accumulate || u0 > 0) ? 1 : 0;
 
-    const dim3 grid(strips, splits, 1), block(waves * WAVE);
-    int rc = INT4MM_OK;
-    if (noting("matvec_kernel<bits=%d,%s,lane_groups=%d,prefetch=%d> strips=%d splits=%d waves=%d units_per_workgroup=%d batch=%d",
-               bits, sparse_mask ? "16:32" : "dense", lk, (int)pf, strips, splits, waves, upwg, (int)B))
-        return INT4MM_OK;
-    for (int64_t b = 0; b < B; ++b) {                      // one pass over the weights per batch row
-        a.outs = (h16*)outs + b * S;
-        a.x = (const h16*)multiplier + b * K;
-        if (sparse_mask) launch<4, true>(a, lk, pf, grid, block, st);
-        else if (bits == 4) launch<4, false>(a, lk, pf, grid, block, st);
-        else if (bits == 3) launch<3, false>(a, lk, pf, grid, block, st);
-        else launch<2, false>(a, lk, pf, grid, block, st);
-        rc = check_launch("matvec");
-        if (rc != INT4MM_OK) return rc;
+        const dim3 grid(strips, splits, 1), block(waves * WAVE);
+        if (noting("matvec_kernel<bits=%d,%s,lane_groups=%d,prefetch=%d> strips=%d splits=%d waves=%d units_per_workgroup=%d batch=%d",
+                   bits, sparse_mask ? "16:32" : "dense", lk, (int)pf, strips, splits, waves, upwg, (int)B))
+            continue;
+        for (int64_t b = 0; b < B; ++b) {                      // one pass over the weights per batch row
+            a.outs = (h16*)outs + b * S;
+            a.x = (const h16*)multiplier + b * K + u0 * 64;
+            if (sparse_mask) launch<4, true>(a, lk, pf, grid, block, st);
+            else if (bits == 4) launch<4, false>(a, lk, pf, grid, block, st);
+            else if (bits == 3) launch<3, false>(a, lk, pf, grid, block, st);
+            else launch<2, false>(a, lk, pf, grid, block, st);
+            const int rc = check_launch("matvec");
+            if (rc != INT4MM_OK) return rc;
+        }
     }
     return INT4MM_OK;
 }
@@ -1156,24 +1128,32 @@ static void* g_scratch_ptr[STATIC_MAX_DEVICES];
 static std::mutex g_scratch_mu;
 }  // namespace i4
 
+// The calling thread's current device's copy of the built-in array (resolved on first use); false if the
+// runtime cannot name it.
+bool i4::static_scratch(void** ptr, size_t* bytes) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= STATIC_MAX_DEVICES) return false;
+    std::lock_guard<std::mutex> lock(g_scratch_mu);
+    if (g_scratch_ptr[dev] == nullptr) {                        // first call on this device
+        void* p = nullptr;
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || p == nullptr) {
+            (void)hipGetLastError();
+            return false;
+        }
+        g_scratch_ptr[dev] = p;
+    }
+    *ptr = g_scratch_ptr[dev];
+    *bytes = STATIC_SCRATCH_BYTES;
+    return true;
+}
+
 extern "C" int int4mm_matvec_static(int bits, void* outs, const void* matrix, const void* multiplier,
                                     const void* scales, const void* zeros, const void* sparse_mask,
                                     const int4mm_shape* shape, void* stream) {
     if (shape == nullptr) return INT4MM_ERR_NULL;
     if (shape->out_size > STATIC_MAX_OUT_SIZE) return INT4MM_ERR_WORKSPACE;     // beyond the built-in scratch
-    int dev = -1;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= STATIC_MAX_DEVICES) return INT4MM_ERR_LAUNCH;
     void* ptr;
-    {
-        std::lock_guard<std::mutex> lock(g_scratch_mu);
-        ptr = g_scratch_ptr[dev];
-        if (ptr == nullptr) {                                   // first call on this device
-            if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || ptr == nullptr) {
-                (void)hipGetLastError();
-                return INT4MM_ERR_LAUNCH;
-            }
-            g_scratch_ptr[dev] = ptr;
-        }
-    }
-    return matvec_impl(bits, outs, matrix, multiplier, scales, zeros, sparse_mask, shape, ptr, STATIC_SCRATCH_BYTES, stream);
+    size_t bytes;
+    if (!static_scratch(&ptr, &bytes)) return INT4MM_ERR_LAUNCH;
+    return matvec_impl(bits, outs, matrix, multiplier, scales, zeros, sparse_mask, shape, ptr, bytes, stream);
 }

@@ -81,15 +81,6 @@ __device__ __forceinline__ uint32_t word_of(const typename Words<CW>::type& v, i
     else return v[c];
 }
 
-// A 32-bit constant kept in a VGPR: VOP3 encodings on this target cannot carry two
-// different literals, so v_and_or_b32 is only selected when mask and magic are
-// registers.  The expression itself stays visible to the compiler, which has to
-// track the VALU -> MFMA operand hazards.
-__device__ __forceinline__ uint32_t vgpr_const(uint32_t literal) {
-    uint32_t r;
-    asm("v_mov_b32 %0, %1" : "=v"(r) : "s"(literal));
-    return r;
-}
 
 // Per format: the k order of the 8 halves of an operand chunk, the offsets the
 // magic-number decode leaves on the low / high half of operand register e, and
@@ -359,11 +350,11 @@ __global__ __launch_bounds__(512) void skinny_kernel(SkinnyArgs a) {
 
         words_t w[PF][NL];
         u32x4 xr[PFX][RT];
-        const uint32_t m0 = vgpr_const(BITS == 4 ? 0x000F000Fu : BITS == 2 ? 0x000C0003u : 0x00380007u);
-        const uint32_t g0 = vgpr_const(BITS == 4 ? 0x64006400u : BITS == 2 ? 0x5C006400u : 0x58006400u);
-        const uint32_t m1 = BITS == 4 ? vgpr_const(0x00F000F0u) : 0u, g1 = BITS == 4 ? vgpr_const(0x54005400u) : 0u;
-        const uint32_t sp_nib = SPARSE ? vgpr_const(0x0F0F0F0Fu) : 0u, sp_flag = SPARSE ? vgpr_const(0x10101010u) : 0u;
-        const uint32_t sp_kept = SPARSE ? vgpr_const(0x00100010u) : 0u, sp_idx = SPARSE ? vgpr_const(0x00000FF0u) : 0u;
+        const uint32_t m0 = in_vgpr(BITS == 4 ? 0x000F000Fu : BITS == 2 ? 0x000C0003u : 0x00380007u);
+        const uint32_t g0 = in_vgpr(BITS == 4 ? 0x64006400u : BITS == 2 ? 0x5C006400u : 0x58006400u);
+        const uint32_t m1 = BITS == 4 ? in_vgpr(0x00F000F0u) : 0u, g1 = BITS == 4 ? in_vgpr(0x54005400u) : 0u;
+        const uint32_t sp_nib = SPARSE ? in_vgpr(0x0F0F0F0Fu) : 0u, sp_flag = SPARSE ? in_vgpr(0x10101010u) : 0u;
+        const uint32_t sp_kept = SPARSE ? in_vgpr(0x00100010u) : 0u, sp_idx = SPARSE ? in_vgpr(0x00000FF0u) : 0u;
         float gS = 0.f, gO = 0.f;           // sums of the current group so far (row lane / 2)
         float nS, nO;                       // sums of the unit staged last (the next to be multiplied)
         // scale / zero of the lane's CW columns for group gi, from the LDS copy
@@ -731,9 +722,9 @@ __global__ __launch_bounds__(512) void wide_rows_kernel(SkinnyArgs a) {
 
     words_t w[PF][NL];
     XRegs xr[PF];
-    const uint32_t m0 = vgpr_const(BITS == 4 ? 0x000F000Fu : BITS == 2 ? 0x000C0003u : 0x00380007u);
-    const uint32_t g0 = vgpr_const(BITS == 4 ? 0x64006400u : BITS == 2 ? 0x5C006400u : 0x58006400u);
-    const uint32_t m1 = BITS == 4 ? vgpr_const(0x00F000F0u) : 0u, g1 = BITS == 4 ? vgpr_const(0x54005400u) : 0u;
+    const uint32_t m0 = in_vgpr(BITS == 4 ? 0x000F000Fu : BITS == 2 ? 0x000C0003u : 0x00380007u);
+    const uint32_t g0 = in_vgpr(BITS == 4 ? 0x64006400u : BITS == 2 ? 0x5C006400u : 0x58006400u);
+    const uint32_t m1 = BITS == 4 ? in_vgpr(0x00F000F0u) : 0u, g1 = BITS == 4 ? in_vgpr(0x54005400u) : 0u;
     h16 sc[CW], ze[CW];
     h16x2 s2[CW], c2[CW];               // {s, s} and {z, z} of the lane's columns
 #pragma unroll
@@ -753,8 +744,8 @@ __global__ __launch_bounds__(512) void wide_rows_kernel(SkinnyArgs a) {
     // ORed with 1024 is 1040 + q; minus 1040 the code, exactly, or -16; then the same two roundings, and
     // the dropped rows are multiplied by 0 -- bit 4 of the half, the "kept" flag, times 0x3C0 is fp16 1.0
     const uint32_t below = SPARSE ? (1u << (8 * h)) - 1u : 0u, rep_h = 0x01010101u * h;
-    const uint32_t sp_nib = SPARSE ? vgpr_const(0x0F0F0F0Fu) : 0u, sp_flag = SPARSE ? vgpr_const(0x10101010u) : 0u;
-    const uint32_t sp_kept = SPARSE ? vgpr_const(0x00100010u) : 0u, sp_idx = SPARSE ? vgpr_const(0x00000FF0u) : 0u;
+    const uint32_t sp_nib = SPARSE ? in_vgpr(0x0F0F0F0Fu) : 0u, sp_flag = SPARSE ? in_vgpr(0x10101010u) : 0u;
+    const uint32_t sp_kept = SPARSE ? in_vgpr(0x00100010u) : 0u, sp_idx = SPARSE ? in_vgpr(0x00000FF0u) : 0u;
     auto sparse_chunk = [&](const words_t w[NL], int blk, int c, uint32_t& v, uint32_t& mb4) {
         const uint32_t m = word_of<CW>(w[3 * blk + 2], c);
         const uint64_t st = ((uint64_t)word_of<CW>(w[3 * blk + 1], c) << 32) | word_of<CW>(w[3 * blk], c);

@@ -23,7 +23,11 @@ def _check(H, p, kind, prior=None):
     d = H.dev_problem(p)
     exact, f32 = H.oracles(p)
     got = H.run_capi(p, d, kind, outs_init=prior)
-    H.assert_product_close(got, exact, f32, prior=prior if kind == "vec" else None, kind="vec")
+    # the kernels that apply scale and zero in fp32 per group are also held to the fp32 oracle on the tight
+    # floor; which kernel serves the call is the launcher's word (it sees this thread's tuning keys too)
+    line = H.capi.describe_launch(kind, p["bits"], p["B"], p["M"], p["K"], p["S"], p["group_size"], p["sparse_mask"] is not None)
+    tight = line.startswith(("skinny_kernel", "matvec_kernel"))
+    H.assert_product_close(got, exact, f32, prior=prior if kind == "vec" else None, kind="vec", tight=tight)
     return d, got
 
 

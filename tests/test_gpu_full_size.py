@@ -35,6 +35,8 @@ def _matvec_against_oracle_by_column_chunks(H, p, got, chunk=2048):
         exact[:, cols] = O.matmul_exact(x, w16)
         w32 = O.dequantize_matrix_fp32(bits, p["matrix"][:, cols], p["scales"][:, cols], p["zeros"][:, cols], g, mask)
         f32[:, cols] = O.matmul_fp32(x, w32)
+    f32 = f32.view(H.OracleArray)
+    f32.bits = bits                                           # (the tight-floor bar depends on the format)
     H.assert_product_close(got.reshape(1, 1, S), exact.reshape(1, 1, S), f32.reshape(1, 1, S))
 
 

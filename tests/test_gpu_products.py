@@ -38,6 +38,25 @@ def test_matvec_parity(H, bits, sparse, K, S, g):
     H.assert_product_close(got2, exact, f32)
 
 
+@pytest.mark.parametrize("bits,sparse,g", [(4, False, 128), (3, False, 256), (4, True, 64), (2, False, -1)])
+def test_matvec_of_a_k_longer_than_one_launch_covers(H, bits, sparse, g):
+    """K = 458752 + 8192: beyond the 32 x 224 units of 64 rows that one launch stages and splits, so the
+    product runs as two launches, the second adding onto the first (the reference's grid covers any K:
+    matvec_kernel.cu:339-347); with a prior in outs and two batch rows"""
+    K = 458752 + 8192
+    p = _problem(bits, sparse, K=K, S=64, M=1, B=2, group_size=g, seed=21)
+    d = H.dev_problem(p)
+    assert H.capi.describe_launch("vec", bits, 1, 1, K, 64, g, sparse).count("matvec_kernel<") == 2
+    exact, f32 = H.oracles(p)
+    prior = np.random.default_rng(2).standard_normal((2, 1, 64)).astype(np.float16)
+    H.capi.tune(5, 1)                    # (the single-row kernel, not the few-row kernel the batch would take)
+    try:
+        got = H.run_capi(p, d, "vec", outs_init=prior)
+    finally:
+        H.capi.tune(5, 0)
+    H.assert_product_close(got, exact, f32, prior=prior)
+
+
 @pytest.mark.parametrize("bits,sparse", FORMATS)
 def test_matvec_accumulates_onto_prior_outs_and_batches(H, bits, sparse):
     p = _problem(bits, sparse, K=512, S=192, M=1, B=3, group_size=64, seed=4)
