@@ -70,6 +70,10 @@ def test_argument_validation_happens_on_the_host():
     assert lib.int4mm_dequantize(4, vp(16), vp(16), vp(16), vp(16), None, 64, 64, 1, 32, None) == 4
     assert lib.int4mm_dequantize(4, None, vp(16), vp(16), vp(16), None, 64, 64, 1, 64, None) == 5
     assert lib.int4mm_workspace_bytes(20480) >= 20480 * 8
+    # a NULL workspace names the array built into the library only together with a size of 0
+    assert lib.int4mm_workspace_status(None, 4096, None) == 5
+    assert lib.int4mm_workspace_init(None, 4096, None) == 5
+    assert lib.int4mm_workspace_init(vp(4096), 16, None) == 6
     assert lib.int4mm_tune(99, 1) != 0 and lib.int4mm_tune(0, 0) == 0
 
 
