@@ -91,7 +91,7 @@ INT4MM_API int int4mm_abi_version(void);
  * shape allows a split at all), 7 = 1: the tiles of a matmul's last, partly
  * filled round are not split, 8 = the few-row kernel whose waves share the
  * staged states: 1 = never, n >= 2 = from n rows on whatever the shape,
- * 9 = unused,
+ * 9 = 1: few-row products never take the balanced launch (workgroups sharing the strips evenly),
  * 10 = polls after which a matvec hand-over gives up (failure-handling tests). */
 INT4MM_API int int4mm_tune(int key, int64_t value);
 

@@ -111,7 +111,7 @@ int int4mm_abi_version(void) { return 1; }
 // 6 = matmul split-K factor (1 = never, 2..8 = forced where the shape allows a split),
 // 7 = 1: the tiles of a matmul's last, partly filled round are not split,
 // 8 = 1: 33 .. 96 rows take the few-row kernel whose waves stage their own states,
-// 9 = unused, 10 = polls before a matvec hand-over gives up.
+// 9 = 1: no balanced few-row launch, 10 = polls before a matvec hand-over gives up.
 int int4mm_tune(int key, int64_t value) {
     if (key < 0 || key >= TUNE_COUNT) return INT4MM_ERR_SHAPE;
     g_tuning[key] = value;

@@ -116,7 +116,7 @@ int validate_product(int bits, const void* outs, const void* matrix, const void*
                      const int4mm_shape* sh, bool matvec);
 int64_t tuning(int key);                       // see int4mm_tune (values are per host thread)
 enum TuneKey { TUNE_MV_WAVES = 0, TUNE_MV_UNITS = 1, TUNE_MV_LK = 2, TUNE_MM_VARIANT = 3, TUNE_MV_NOPF = 4,
-               TUNE_NO_SKINNY = 5, TUNE_MM_SPLIT = 6, TUNE_MM_TAIL = 7, TUNE_NO_WIDE = 8, TUNE_RESERVED_9 = 9,
+               TUNE_NO_SKINNY = 5, TUNE_MM_SPLIT = 6, TUNE_MM_TAIL = 7, TUNE_NO_WIDE = 8, TUNE_NO_BALANCE = 9,
                TUNE_MV_SPIN = 10, TUNE_COUNT = 11 };
 
 // int4mm_describe_launch: while this thread is "noting", a launcher records the kernel and launch

@@ -64,6 +64,11 @@ struct SkinnyArgs {
     float* part;
     int* counters;
     int block_rows;         // wide kernel: rows of states per workgroup (blockIdx.y), a multiple of 16
+    // balanced launch of the few-row kernel (more strips than CUs): `bal_wgs` workgroups share the strips' units
+    // evenly, workgroup i takes [i q + i r / wgs, (i + 1) q + (i + 1) r / wgs) of strips x units, strip-major
+    int bal_wgs, bal_q, bal_r;
+    // launch with a fifth column per lane: the first `wide_wgs` workgroups take 80 columns, the others 64
+    int wide_wgs;
 };
 
 constexpr int SK_PITCH = 144;                   // bytes between rows of a staged unit (128 + 16: conflict-free)
@@ -175,24 +180,127 @@ __device__ __forceinline__ h16x8 exact_operand(uint32_t f, uint32_t m0, uint32_t
     return bitcast<h16x8>(r);
 }
 
+// Balanced launch: workgroup i of `wgs` takes the range [i q + i r / wgs, (i + 1) q + (i + 1) r / wgs) of
+// strips x units (strip-major; q, r = quotient and remainder of the total by wgs).  The range is at least one
+// strip and less than two strips long, so it touches at most three strips: three segments, segment k on strip
+// strip0 + k.  The workgroup's waves are dealt to the segments in proportion to their units (at least one each).
+// For one wave: its segment (`mine`), the segment's units [lo, hi) within its strip, the segment's first wave
+// and number of waves; for the workgroup's copy of scales and zeros in LDS: the first group of each segment
+// and where each segment's groups start (goff3: all groups).
+struct BalancedShare { int strip0, mine, lo, hi, wave0, waves, glo0, glo1, glo2, goff1, goff2, goff3; };
+// a / b for 0 <= a < 2^22, b >= 1 through the float reciprocal (one step of correction either way): a dozen such
+// quotients stand between a wave's start and its first loads, and the compiler's exact division is ~35 instructions
+__device__ __forceinline__ int small_div(int a, int b, float inv_b) {
+    int q = (int)((float)a * inv_b);
+    int r = a - q * b;
+    if (r < 0) { --q; r += b; }
+    if (r >= b) ++q;
+    return q;
+}
+__device__ __forceinline__ BalancedShare balanced_share(int q, int r, int i, int units, int group_units, int nwaves, int wave) {
+    BalancedShare b{};
+    constexpr int WGS = 256;                                         // (SK_BAL_WGS, the host side's constant)
+    const int lo = i * q + ((i * r) >> 8), hi = (i + 1) * q + (((i + 1) * r) >> 8);
+    const int share = hi - lo;
+    static_assert(WGS == 1 << 8, "the shifts above");
+    const float inv_units = 1.f / (float)units, inv_gu = 1.f / (float)group_units, inv_share = 1.f / (float)share;
+    b.strip0 = small_div(lo, units, inv_units);
+    int seg_lo[3], seg_n[3], seg_w[3], dealt = 0;
+#pragma unroll
+    for (int k = 0; k < 3; ++k) {
+        const int s0 = (b.strip0 + k) * units;
+        const int from = max(lo, s0), to = min(hi, s0 + units);
+        seg_lo[k] = from - s0;
+        seg_n[k] = max(0, to - from);
+        seg_w[k] = seg_n[k] > 0 ? max(1, small_div(seg_n[k] * nwaves + share / 2, share, inv_share)) : 0;
+        dealt += seg_w[k];
+    }
+    // the rounding may deal a wave or two too many or too few: take from the segment with the fewest units per
+    // wave, give to the one with the most (the pick's units and waves are kept by value: no indexed registers)
+#pragma unroll
+    for (int it = 0; it < 3; ++it) {
+        if (dealt > nwaves) {
+            int k = -1, kn = 0, kw = 1;
+#pragma unroll
+            for (int c = 0; c < 3; ++c)
+                if (seg_w[c] > 1 && (k < 0 || seg_n[c] * kw < kn * seg_w[c])) { k = c; kn = seg_n[c]; kw = seg_w[c]; }
+#pragma unroll
+            for (int c = 0; c < 3; ++c) if (c == k) --seg_w[c];
+            --dealt;
+        } else if (dealt < nwaves) {
+            int k = -1, kn = 0, kw = 1;
+#pragma unroll
+            for (int c = 0; c < 3; ++c)
+                if (seg_n[c] > 0 && (k < 0 || seg_n[c] * kw > kn * seg_w[c])) { k = c; kn = seg_n[c]; kw = seg_w[c]; }
+#pragma unroll
+            for (int c = 0; c < 3; ++c) if (c == k) ++seg_w[c];
+            ++dealt;
+        }
+    }
+    int w0 = 0;
+#pragma unroll
+    for (int k = 0; k < 3; ++k) {
+        if (wave >= w0 && wave < w0 + seg_w[k]) { b.mine = k; b.wave0 = w0; b.waves = seg_w[k]; b.lo = seg_lo[k]; b.hi = seg_lo[k] + seg_n[k]; }
+        w0 += seg_w[k];
+    }
+    const int g0 = small_div(seg_lo[0], group_units, inv_gu), g1 = small_div(seg_lo[1], group_units, inv_gu),
+              g2 = small_div(seg_lo[2], group_units, inv_gu);
+    b.glo0 = g0; b.glo1 = g1; b.glo2 = g2;
+    b.goff1 = seg_n[0] > 0 ? small_div(seg_lo[0] + seg_n[0] - 1, group_units, inv_gu) + 1 - g0 : 0;
+    b.goff2 = b.goff1 + (seg_n[1] > 0 ? small_div(seg_lo[1] + seg_n[1] - 1, group_units, inv_gu) + 1 - g1 : 0);
+    b.goff3 = b.goff2 + (seg_n[2] > 0 ? small_div(seg_lo[2] + seg_n[2] - 1, group_units, inv_gu) + 1 - g2 : 0);
+    return b;
+}
+
 // CW: columns per lane; RT: row groups of 8 that can hold real rows (R <= 8 RT);
 // MT: 16-row MFMA tiles; PF: units of packed weights in flight per wave
-template <int BITS, int CW, int RT, bool SPARSE>
+// BAL: the workgroups share the work evenly instead of taking a strip each (more strips than CUs): a workgroup's
+// range of (strip, unit) touches two or three strips, its waves are dealt to them in proportion, every wave works
+// on one strip, and a strip that two workgroups share is summed through the hand-over below.
+// XC = 1: a fifth column per lane (CW = 4 only, dense formats): the workgroup's columns are four or five slivers of
+// 16, the lane's four adjacent columns in the first four and column j of the fifth (a.wide_wgs workgroups have one)
+template <int BITS, int CW, int RT, bool SPARSE, bool BAL = false, int XC = 0>
 __global__ __launch_bounds__(512) void skinny_kernel(SkinnyArgs a) {
     using F = SkFmt<BITS, SPARSE>;
     constexpr int NL = F::LOADS;
     constexpr int PF = (BITS == 3 && CW == 4) || (SPARSE && CW == 4) ? 2 : 4, MT = RT == 4 ? 2 : 1;
     constexpr int PFX = RT == 4 ? 2 : 4;            // units of states in flight per wave
-    constexpr int STRIP = 16 * CW;
+    constexpr int CT = CW + XC;                     // columns per lane in all
+    constexpr int STRIP = 16 * CT;
     extern __shared__ __attribute__((aligned(16))) char lds[];
     typedef typename Words<CW>::type words_t;
     const int t = threadIdx.x, lane = t & 63, nwaves = blockDim.x >> 6;
     const int wave = __builtin_amdgcn_readfirstlane(t >> 6);   // scalar: the unit loop runs on SGPRs
     const int j = lane & 15, h = lane >> 4;
-    const int col0 = blockIdx.x * STRIP + CW * j;              // first of this lane's CW columns
     const int units = a.K / 64;
-    const int split_lo = blockIdx.z * a.units_per_split, split_hi = min(units, split_lo + a.units_per_split);
-    const int u0 = min(split_hi, split_lo + wave * a.units_per_wave), u1 = min(split_hi, u0 + a.units_per_wave);
+    // the wave's strip, the part of the strip's units that its workgroup (BAL: its segment of the workgroup's
+    // range) covers, and the wave's own units in it
+    int strip = blockIdx.x, split_lo, split_hi, u0, u1;
+    int seg_wave0 = 0, seg_waves = nwaves;                      // the waves that work on the same strip
+    BalancedShare bs{};
+    if constexpr (BAL) {
+        bs = balanced_share(a.bal_q, a.bal_r, blockIdx.x, units, a.group_units, nwaves, wave);
+        strip = bs.strip0 + bs.mine;
+        split_lo = bs.lo;
+        split_hi = bs.hi;
+        seg_wave0 = bs.wave0;
+        seg_waves = bs.waves;
+        const int upw = small_div(split_hi - split_lo + seg_waves - 1, seg_waves, 1.f / (float)seg_waves);
+        u0 = min(split_hi, split_lo + (wave - seg_wave0) * upw);
+        u1 = min(split_hi, u0 + upw);
+    } else {
+        split_lo = blockIdx.z * a.units_per_split;
+        split_hi = min(units, split_lo + a.units_per_split);
+        u0 = min(split_hi, split_lo + wave * a.units_per_wave);
+        u1 = min(split_hi, u0 + a.units_per_wave);
+    }
+    // first column of the workgroup, of the lane's CW adjacent columns, and the lane's column in the fifth sliver
+    // (a workgroup without one re-reads its first sliver there and does not write the result)
+    const bool has_extra = XC != 0 && (int)blockIdx.x < a.wide_wgs;
+    const int colbase = XC != 0 ? (has_extra ? 80 * (int)blockIdx.x : 80 * a.wide_wgs + 64 * ((int)blockIdx.x - a.wide_wgs))
+                                : strip * STRIP;
+    const int col0 = colbase + CW * j;
+    const int colx = has_extra ? colbase + 16 * CW + j : colbase + j;
     // more than 32 rows: blockIdx.y takes rows 32 y .. 32 y + 31 (each block reads the strip's weights again)
     const int row0 = blockIdx.y * 32;
     const int R = min(32, a.R - row0);
@@ -205,6 +313,8 @@ __global__ __launch_bounds__(512) void skinny_kernel(SkinnyArgs a) {
     // (of the groups that the workgroup's share of K touches: group_lo onwards)
     const int group_lo = split_lo / a.group_units;
     const int groups = (split_hi + a.group_units - 1) / a.group_units - group_lo;
+    // (BAL: the copies of the workgroup's segments one after the other; this wave's starts at group sz_goff)
+    const int sz_groups = BAL ? bs.goff3 : groups, sz_goff = BAL ? (bs.mine == 0 ? 0 : bs.mine == 1 ? bs.goff1 : bs.goff2) : 0;
     // (16:32: the selector table is allocated statically: its LDS address is a compile-time constant)
     __shared__ __attribute__((aligned(16))) u32x4 lut_table[SPARSE ? 256 : 1];
     const char* lut = reinterpret_cast<const char*>(lut_table);
@@ -228,15 +338,25 @@ __global__ __launch_bounds__(512) void skinny_kernel(SkinnyArgs a) {
         }
     }
     uint32_t* sz = reinterpret_cast<uint32_t*>(lds + nwaves * SK_WAVE_LDS + 16);      // scales, then zeros
-    auto scan_scales = [&]() -> bool {
+    auto scan_scales = [&]() __attribute__((always_inline)) -> bool {
         int* flag = reinterpret_cast<int*>(lds + nwaves * SK_WAVE_LDS);
         if (t == 0) *flag = 0;
         __syncthreads();
         bool bad = false;
-        const int n = groups * (STRIP / 2);
+        const int n = sz_groups * (STRIP / 2);
         for (int i = t; i < n; i += blockDim.x) {
             const int g = i / (STRIP / 2), c = i % (STRIP / 2);
-            const int64_t at = (int64_t)(group_lo + g) * a.S + blockIdx.x * STRIP + 2 * c;
+            int64_t at;
+            if constexpr (BAL) {
+                // (sums rather than selections among the three segments' values: the compiler turns a selection
+                // among fields into an indexed load, which puts the whole record into scratch memory)
+                const int k1 = g >= bs.goff1 ? 1 : 0, k2 = g >= bs.goff2 ? 1 : 0;
+                const int first = bs.glo0 + k1 * (bs.glo1 - bs.glo0) + k2 * (bs.glo2 - bs.glo1);
+                const int off = k1 * bs.goff1 + k2 * (bs.goff2 - bs.goff1);
+                at = (int64_t)(first + g - off) * a.S + (bs.strip0 + k1 + k2) * STRIP + 2 * c;
+            } else {
+                at = (int64_t)(group_lo + g) * a.S + colbase + ((XC != 0 && !has_extra && c >= 8 * CW) ? 2 * c - 16 * CW : 2 * c);
+            }
             const uint32_t two = *reinterpret_cast<const uint32_t*>(a.scales + at);
             bad |= !(as_h2(two).x >= (h16)0.0f) || !(as_h2(two).y >= (h16)0.0f);
             sz[i] = two;
@@ -254,9 +374,9 @@ __global__ __launch_bounds__(512) void skinny_kernel(SkinnyArgs a) {
     // accumulators: acc = raw products of the current group, y = finished groups
     // (register e of tile mt is row 16 mt + 4 h + e, column j)
     // (16:32: accm = the same for the "kept" flags)
-    f32x4 acc[CW][MT], accm[SPARSE ? CW : 1][MT], y[CW][MT];
+    f32x4 acc[CT][MT], accm[SPARSE ? CW : 1][MT], y[CT][MT];
 #pragma unroll
-    for (int c = 0; c < CW; ++c)
+    for (int c = 0; c < CT; ++c)
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
             acc[c][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -278,7 +398,8 @@ __global__ __launch_bounds__(512) void skinny_kernel(SkinnyArgs a) {
         //          (w[3 blk], w[3 blk + 1], w[3 blk + 2])
         const uint32_t* wbase = a.matrix + (int64_t)(SPARSE ? 0 : wrow) * a.S + col0;
         const uint32_t* mbase = SPARSE ? a.mask + col0 : nullptr;
-        auto load_w = [&](words_t w[NL], int u) {
+        const uint32_t* xbase = a.matrix + (int64_t)wrow * a.S + colx;
+        auto load_w = [&](words_t w[NL], uint32_t wx[NL], int u) {
             const uint32_t* p = wbase + (int64_t)u * (2 * F::ROWS) * a.S;
             if constexpr (SPARSE) {
                 const uint32_t* pm = mbase + (int64_t)u * 2 * a.S;
@@ -293,17 +414,20 @@ __global__ __launch_bounds__(512) void skinny_kernel(SkinnyArgs a) {
                 for (int i = 0; i < NL; ++i) {
                     const int row = BITS == 3 ? 3 * (i >> 1) + (i & 1) : F::ROWS * i;       // relative to the lane's first row
                     w[i] = __builtin_nontemporal_load(reinterpret_cast<const words_t*>(p + (int64_t)row * a.S));
+                    if constexpr (XC != 0)
+                        wx[i] = __builtin_nontemporal_load(xbase + ((int64_t)u * (2 * F::ROWS) + row) * a.S);
                 }
             }
         };
         // 16:32: mask bits of the rows before the lane group's eight; selector that replicates mask byte h
         const uint32_t below = SPARSE ? (1u << (8 * h)) - 1u : 0u, rep_h = 0x01010101u * h;
         // the 8 codes of chunk h of block blk, column c
-        auto chunk_bits = [&](const words_t w[NL], int blk, int c) -> uint32_t {
+        auto chunk_bits = [&](const words_t w[NL], const uint32_t wx[NL], int blk, int c) -> uint32_t {
+            auto word = [&](int idx) -> uint32_t { return c < CW ? word_of<CW>(w[idx], c < CW ? c : 0) : wx[idx]; };
             if constexpr (BITS == 3)
-                return (uint32_t)((((uint64_t)word_of<CW>(w[2 * blk + 1], c) << 32) | word_of<CW>(w[2 * blk], c)) >> wshift);
+                return (uint32_t)((((uint64_t)word(2 * blk + 1) << 32) | word(2 * blk)) >> wshift);
             else
-                return word_of<CW>(w[blk], c) >> wshift;
+                return word(blk) >> wshift;
         };
         // states of unit u (8 RT rows x 128 bytes): 8 / RT lanes per row, RT 16-byte chunks
         // each; the rows of the LDS buffers beyond 8 RT stay zero
@@ -349,6 +473,7 @@ __global__ __launch_bounds__(512) void skinny_kernel(SkinnyArgs a) {
         for (int i = lane; i < 2 * SK_XBUF / 16; i += 64) *reinterpret_cast<u32x4*>(my + i * 16) = u32x4{0, 0, 0, 0};
 
         words_t w[PF][NL];
+        uint32_t wx[PF][NL];                // (XC: the fifth column's words)
         u32x4 xr[PFX][RT];
         const uint32_t m0 = in_vgpr(BITS == 4 ? 0x000F000Fu : BITS == 2 ? 0x000C0003u : 0x00380007u);
         const uint32_t g0 = in_vgpr(BITS == 4 ? 0x64006400u : BITS == 2 ? 0x5C006400u : 0x58006400u);
@@ -358,12 +483,12 @@ __global__ __launch_bounds__(512) void skinny_kernel(SkinnyArgs a) {
         float gS = 0.f, gO = 0.f;           // sums of the current group so far (row lane / 2)
         float nS, nO;                       // sums of the unit staged last (the next to be multiplied)
         // scale / zero of the lane's CW columns for group gi, from the LDS copy
-        h16 sc[CW], ze[CW];
+        h16 sc[CT], ze[CT];
 #pragma unroll
-        for (int c = 0; c < CW; ++c) { sc[c] = (h16)0.f; ze[c] = (h16)0.f; }
+        for (int c = 0; c < CT; ++c) { sc[c] = (h16)0.f; ze[c] = (h16)0.f; }
         auto load_sz = [&](int gi) {
-            const h16* ps = reinterpret_cast<const h16*>(sz) + (gi - group_lo) * STRIP + CW * j;
-            const h16* pz = ps + groups * STRIP;
+            const h16* ps = reinterpret_cast<const h16*>(sz) + (sz_goff + gi - group_lo) * STRIP + CW * j;
+            const h16* pz = ps + sz_groups * STRIP;
             if constexpr (CW == 4) {
                 const u32x2 s2 = *reinterpret_cast<const u32x2*>(ps), z2 = *reinterpret_cast<const u32x2*>(pz);
                 sc[0] = as_h2(s2.x).x; sc[1] = as_h2(s2.x).y; sc[2] = as_h2(s2.y).x; sc[3] = as_h2(s2.y).y;
@@ -374,10 +499,11 @@ __global__ __launch_bounds__(512) void skinny_kernel(SkinnyArgs a) {
             } else {
                 sc[0] = ps[0]; ze[0] = pz[0];
             }
+            if constexpr (XC != 0) { sc[CW] = ps[16 * CW + j - CW * j]; ze[CW] = pz[16 * CW + j - CW * j]; }
         };
 
 #pragma unroll
-        for (int f = 0; f < PF; ++f) load_w(w[f], min(u0 + f, u1 - 1));
+        for (int f = 0; f < PF; ++f) load_w(w[f], wx[f], min(u0 + f, u1 - 1));
         load_x(xr[0], u0);
         general = scan_scales();
         stage_x(xr[0], 0, nS, nO);
@@ -387,7 +513,7 @@ __global__ __launch_bounds__(512) void skinny_kernel(SkinnyArgs a) {
 
         // p: parity of the LDS buffer that holds unit u; xn: the register set with the states of unit u + 1.
         // The decode mode is a compile-time tag: one loop body per mode, no branches inside.
-        auto step = [&](auto mode, int u, int p, words_t w[NL], u32x4 xn[RT]) {
+        auto step = [&](auto mode, int u, int p, words_t w[NL], uint32_t wx[NL], u32x4 xn[RT]) {
             constexpr bool general = decltype(mode)::value;
             if constexpr (general) {
                 if (u == u0 || u % a.group_units == 0) load_sz(u / a.group_units);
@@ -401,7 +527,7 @@ __global__ __launch_bounds__(512) void skinny_kernel(SkinnyArgs a) {
                 for (int mt = 0; mt < MT; ++mt)
                     xa[mt] = *reinterpret_cast<const h16x8*>(my + p * SK_XBUF + (j + 16 * mt) * SK_PITCH + (i * 4 + h) * 16);
 #pragma unroll
-                for (int c = 0; c < CW; ++c) {
+                for (int c = 0; c < CT; ++c) {
                     if constexpr (SPARSE) {
                         const uint32_t m = word_of<CW>(w[3 * i + 2], c);
                         const uint64_t st = ((uint64_t)word_of<CW>(w[3 * i + 1], c) << 32) | word_of<CW>(w[3 * i], c);
@@ -426,7 +552,7 @@ __global__ __launch_bounds__(512) void skinny_kernel(SkinnyArgs a) {
                             }
                         }
                     } else {
-                        const uint32_t f = chunk_bits(w, i, c);
+                        const uint32_t f = chunk_bits(w, wx, i, c);
                         const h16x8 wb = general ? exact_operand<BITS>(f, m0, m1, g0, g1, sc[c], ze[c])
                                                  : magic_operand<BITS>(f, m0, m1, g0, g1);
 #pragma unroll
@@ -436,7 +562,7 @@ __global__ __launch_bounds__(512) void skinny_kernel(SkinnyArgs a) {
                 }
             }
             // refill this register set PF units ahead; move the next unit's states to LDS
-            load_w(w, min(u + PF, u1 - 1));
+            load_w(w, wx, min(u + PF, u1 - 1));
             stage_x(xn, p ^ 1, nS, nO);
             load_x(xn, min(u + 1 + PFX, u1 - 1));
             // group complete (or this wave's range ends): fold it into y
@@ -465,7 +591,7 @@ __global__ __launch_bounds__(512) void skinny_kernel(SkinnyArgs a) {
                     const f32x4 s4 = *reinterpret_cast<const f32x4*>(&sums[16 * mt + 4 * h]);
                     const f32x4 o4 = *reinterpret_cast<const f32x4*>(&sums[32 + 16 * mt + 4 * h]);
 #pragma unroll
-                    for (int c = 0; c < CW; ++c) {
+                    for (int c = 0; c < CT; ++c) {
                         const float sf = general ? 1.f : (float)sc[c];
                         const float z = general ? 0.f : (float)ze[c];
 #pragma unroll
@@ -486,7 +612,7 @@ __global__ __launch_bounds__(512) void skinny_kernel(SkinnyArgs a) {
 #pragma unroll
                 for (int f = 0; f < UN; ++f) {
                     if (f > 0 && u + f >= u1) break;
-                    step(mode, u + f, f & 1, w[f % PF], xr[(f + 1) % PFX]);
+                    step(mode, u + f, f & 1, w[f % PF], wx[f % PF], xr[(f + 1) % PFX]);
                 }
             }
         };
@@ -498,8 +624,29 @@ __global__ __launch_bounds__(512) void skinny_kernel(SkinnyArgs a) {
     __syncthreads();
     constexpr int TILE = MT * 16 * STRIP;
     float* red = reinterpret_cast<float*>(lds);
-    auto tile_at = [&](float* base, int mt, int e) { return base + ((mt * 16 + 4 * h + e) * 16 + j) * CW; };
-    for (int s = nwaves >> 1; s >= 1; s >>= 1) {
+    auto tile_at = [&](float* base, int mt, int e) { return base + ((mt * 16 + 4 * h + e) * 16 + j) * CT; };
+    if constexpr (BAL) {
+        // every wave leaves its tile; the first wave of each segment adds up its segment's, in wave order
+        float* dst = red + wave * TILE;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+#pragma unroll
+                for (int c = 0; c < CT; ++c) tile_at(dst, mt, e)[c] = y[c][mt][e];
+        __syncthreads();
+        if (wave != seg_wave0) return;
+        for (int w = seg_wave0 + 1; w < seg_wave0 + seg_waves; ++w) {
+            float* src = red + w * TILE;
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+#pragma unroll
+                    for (int c = 0; c < CT; ++c) y[c][mt][e] += tile_at(src, mt, e)[c];
+        }
+    }
+    for (int s = BAL ? 0 : (nwaves >> 1); s >= 1; s >>= 1) {
         if (wave >= s && wave < 2 * s) {
             float* dst = red + (wave - s) * TILE;
 #pragma unroll
@@ -507,7 +654,7 @@ __global__ __launch_bounds__(512) void skinny_kernel(SkinnyArgs a) {
 #pragma unroll
                 for (int e = 0; e < 4; ++e)
 #pragma unroll
-                    for (int c = 0; c < CW; ++c) tile_at(dst, mt, e)[c] = y[c][mt][e];
+                    for (int c = 0; c < CT; ++c) tile_at(dst, mt, e)[c] = y[c][mt][e];
         }
         __syncthreads();
         if (wave < s) {
@@ -517,21 +664,24 @@ __global__ __launch_bounds__(512) void skinny_kernel(SkinnyArgs a) {
 #pragma unroll
                 for (int e = 0; e < 4; ++e)
 #pragma unroll
-                    for (int c = 0; c < CW; ++c) y[c][mt][e] += tile_at(src, mt, e)[c];
+                    for (int c = 0; c < CT; ++c) y[c][mt][e] += tile_at(src, mt, e)[c];
         }
         __syncthreads();
     }
-    if (wave == 0) {
-        if (gridDim.z > 1) {
+    if (BAL || wave == 0) {
+        // (BAL: a strip shared by two workgroups -- never more: a workgroup's range is at least a strip long)
+        const bool shared = BAL ? (split_lo > 0 || split_hi < units) : gridDim.z > 1;
+        if (shared) {
             // hand-over between the workgroups of a strip: write-through stores of the partial tile
             // (value v of lane l at (v * 64 + l) * 4), a device-scope counter, and whoever finds all
             // the others counted reads every partial back in split order -- one summation order
             // whoever is last -- and goes on to write the strip.  One wave: no barrier involved.
             constexpr int NV = CW * MT * 4, THROUGH = 17;                 // sc0 | sc1: straight to memory
-            const int tile = blockIdx.y * gridDim.x + blockIdx.x, ks = gridDim.z;
+            const int tile = BAL ? strip : blockIdx.y * gridDim.x + blockIdx.x, ks = BAL ? 2 : gridDim.z;
+            const int my_split = BAL ? (split_lo > 0 ? 1 : 0) : blockIdx.z;
             char* const slots = reinterpret_cast<char*>(a.part) + (int64_t)tile * ks * (NV * 256);
             const __amdgpu_buffer_rsrc_t mine = __builtin_amdgcn_make_buffer_rsrc(
-                slots + (int64_t)blockIdx.z * (NV * 256), 0, NV * 256, 0x00020000);
+                slots + (int64_t)my_split * (NV * 256), 0, NV * 256, 0x00020000);
 #pragma unroll
             for (int c = 0; c < CW; ++c)
 #pragma unroll
@@ -581,6 +731,12 @@ __global__ __launch_bounds__(512) void skinny_kernel(SkinnyArgs a) {
                         float v = y[c][mt][e];
                         if (a.accumulate) v += (float)o[c];
                         o[c] = (h16)v;
+                    }
+                    if (XC != 0 && has_extra) {
+                        h16* ox = a.outs + (int64_t)(row0 + m) * a.S + colx;
+                        float v = y[CT - 1][mt][e];
+                        if (a.accumulate) v += (float)ox[0];
+                        ox[0] = (h16)v;
                     }
                 }
             }
@@ -1118,6 +1274,100 @@ static bool launch_skinny(const SkinnyArgs& a, int waves, int ksplit, hipStream_
     return true;
 }
 
+// The balanced launch: 64-column strips, eight waves, `wgs` workgroups that share strips x units evenly.
+// Partial tiles of the strips that two workgroups share: two slots per strip in `part`, one counter per strip.
+constexpr int SK_BAL_WGS = 256;
+static size_t skinny_balanced_part_bytes(int64_t S) { return (size_t)(S / 64) * 2 * (4 * 2 * 4 * 256); }
+// Where it pays (8 and 16 rows, K = 3072 ... 14336, us, a workgroup per strip / shared): int4 K=5120, S=20480 19.1 / 16.6,
+// K=8192, S=18432 27.4 / 21.0, K=3072, S=20480 13.8 / 12.9; 16:32 K=5120, S=20480 29.5 / 24.5, K=8192, S=18432 43.5 / 31.0;
+// beyond a quarter more strips than CUs only on a long K, where a workgroup per strip means eight waves each and two
+// rounds (K=12288, S=28672 48.5 / 39.8, K=10240, S=24576 39.0 / 30.9; K=8192, S=22016 28.7 / 29.3 and K=4096, S=28672
+// 17.2 / 18.0 do not gain).  17 ... 32 rows, whose accumulators fill the register file, lose (K=2048, S=20480 14.8 / 15.9).
+static bool balanced_shape(int64_t R, int64_t K, int64_t S) {
+    const int64_t strips = S / 64, units = K / 64;
+    if (R < 2 || R > 16 || S % 64 != 0 || strips <= SK_BAL_WGS || strips >= 2 * SK_BAL_WGS || strips * units >= (1ll << 22)) return false;
+    return units >= (strips <= SK_BAL_WGS * 5 / 4 ? 48 : 160);
+}
+template <int BITS, bool SPARSE>
+static bool launch_skinny_balanced(SkinnyArgs a, hipStream_t st) {
+    constexpr int CW = 4, WAVES = 8;
+    const int strips = a.S / 64, units = a.K / 64;
+    const int rt = (a.R + 7) / 8;
+    const int64_t total = (int64_t)strips * units;
+    a.bal_wgs = SK_BAL_WGS;
+    a.bal_q = (int)(total / SK_BAL_WGS);
+    a.bal_r = (int)(total % SK_BAL_WGS);
+    // scales in LDS: a workgroup's range is less than two strips long and touches at most three
+    const int groups = 2 * ((units + a.group_units - 1) / a.group_units) + 3;
+    size_t lds = (size_t)WAVES * SK_WAVE_LDS + 16 + (size_t)groups * 16 * CW * 4;
+    const size_t red = (size_t)WAVES * 16 * 16 * CW * 4;
+    if (red > lds) lds = red;
+    if (lds > 150 * 1024 - (SPARSE ? 4096 : 0)) return false;
+    const dim3 grid(SK_BAL_WGS, 1, 1), block(WAVES * 64);
+    if (noting("skinny_kernel<bits=%d,%s,columns_per_lane=%d,row_tiles=%d,balanced> strips=%d row_blocks=1 workgroups=%d waves=%d",
+               BITS, SPARSE ? "16:32" : "dense", CW, rt <= 1 ? 1 : 2, strips, SK_BAL_WGS, WAVES))
+        return true;
+    auto go = [&](auto kernel) {
+        static std::atomic<uint64_t> done;
+        int dev = 0;
+        hipGetDevice(&dev);
+        const uint64_t bit = 1ull << (dev & 63);
+        if (!(done.load(std::memory_order_relaxed) & bit)) {
+            hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                150 * 1024);
+            done.fetch_or(bit, std::memory_order_relaxed);
+        }
+        hipLaunchKernelGGL(kernel, grid, block, lds, st, a);
+    };
+    if (rt <= 1) go(skinny_kernel<BITS, CW, 1, SPARSE, true>);
+    else go(skinny_kernel<BITS, CW, 2, SPARSE, true>);            // (up to 16 rows: balanced_shape)
+    return true;
+}
+
+// Between 256 and 320 strips of 64 columns: 256 workgroups of four or five slivers of 16 columns each, so that
+// every CU has one workgroup and none a second (dense formats, up to 16 rows).
+// int3 and int2 (8 and 16 rows, us, a workgroup per strip / shared strips / slivers): K=5120, S=20480 int3 22.5 / 19.3 / 17.8,
+// int2 21.2 / 18.2 / 16.6; K=8192, S=18432 int3 32.4 / 24.1 / 24.2; K=14336, S=19200 int3 56.2 / 44.8 / 38.8, int2 53.0 / 41.3 /
+// 34.6.  int4, whose words carry a third more bytes per unit, does better with shared strips (K=5120, S=20480 18.5 with
+// slivers), and so does 16:32, which has no registers for a fifth column.
+static bool sliver_shape(int bits, int64_t R, int64_t K, int64_t S, bool sparse) {
+    const int64_t slivers = S / 16;
+    return !sparse && bits != 4 && R >= 2 && R <= 16 && S % 64 == 0 && slivers > 4 * SK_BAL_WGS && slivers <= 5 * SK_BAL_WGS &&
+           K / 64 >= 48;
+}
+template <int BITS>
+static bool launch_skinny_slivers(SkinnyArgs a, hipStream_t st) {
+    constexpr int CW = 4, CT = 5, WAVES = 8;
+    const int rt = (a.R + 7) / 8;
+    a.wide_wgs = a.S / 16 - 4 * SK_BAL_WGS;
+    a.units_per_split = a.K / 64;
+    a.units_per_wave = (a.units_per_split + WAVES - 1) / WAVES;
+    const int groups = (a.K / 64 + a.group_units - 1) / a.group_units;
+    size_t lds = (size_t)WAVES * SK_WAVE_LDS + 16 + (size_t)groups * 16 * CT * 4;
+    const size_t red = (size_t)(WAVES / 2) * 16 * 16 * CT * 4;
+    if (red > lds) lds = red;
+    if (lds > 150 * 1024) return false;
+    const dim3 grid(SK_BAL_WGS, 1, 1), block(WAVES * 64);
+    if (noting("skinny_kernel<bits=%d,dense,columns_per_lane=4+1,row_tiles=%d> strips=%d (%d of 80 columns, the others of 64) "
+               "row_blocks=1 ksplit=1 waves=%d", BITS, rt <= 1 ? 1 : 2, SK_BAL_WGS, a.wide_wgs, WAVES))
+        return true;
+    auto go = [&](auto kernel) {
+        static std::atomic<uint64_t> done;
+        int dev = 0;
+        hipGetDevice(&dev);
+        const uint64_t bit = 1ull << (dev & 63);
+        if (!(done.load(std::memory_order_relaxed) & bit)) {
+            hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                150 * 1024);
+            done.fetch_or(bit, std::memory_order_relaxed);
+        }
+        hipLaunchKernelGGL(kernel, grid, block, lds, st, a);
+    };
+    if (rt <= 1) go(skinny_kernel<BITS, CW, 1, false, false, 1>);
+    else go(skinny_kernel<BITS, CW, 2, false, false, 1>);
+    return true;
+}
+
 template <int BITS, bool SPARSE = false>
 static bool launch_skinny_cw(const SkinnyArgs& a, int cw, int waves, int ksplit, hipStream_t st) {
     if (cw == 4) return launch_skinny<BITS, 4, SPARSE>(a, waves, ksplit, st);
@@ -1186,7 +1436,8 @@ size_t skinny_workspace_bytes(int64_t R, int64_t K, int64_t S, bool sparse) {
         const WidePlan w = plan_wide(R, K, S, sparse, group_units);
         if (w.use) wide = std::max(wide, w.part_bytes);
     }
-    return std::max<size_t>(p.ksplit > 1 ? p.part_bytes : 0, wide);
+    const size_t balanced = balanced_shape(R, K, S) ? skinny_balanced_part_bytes(S) : 0;
+    return std::max(std::max<size_t>(p.ksplit > 1 ? p.part_bytes : 0, wide), balanced);
 }
 
 // Product of 2 <= R <= 96 rows with a dense or (sparse_mask != nullptr) 16:32 sparse int4 matrix; beyond that
@@ -1206,6 +1457,8 @@ bool skinny_rows(int bits, h16* outs, const uint32_t* matrix, const h16* x, cons
     a.block_rows = 32;
     a.part = nullptr;
     a.counters = nullptr;
+    a.bal_wgs = 0; a.bal_q = 0; a.bal_r = 0;
+    a.wide_wgs = 0;
     // 33 rows and more, dense: the kernel whose waves share the staged states
     {
         const WidePlan wp = plan_wide(R, K, S, sparse_mask != nullptr, a.group_units);
@@ -1255,6 +1508,25 @@ bool skinny_rows(int bits, h16* outs, const uint32_t* matrix, const h16* x, cons
         if (launch(sp.cw, 8, ksplit)) return true;
     }
     a.units_per_split = units;
+    // a quarter more 64-column strips than CUs at most: a workgroup per CU, of 64 or 80 columns
+    if (tuning(TUNE_NO_BALANCE) == 0 && tuning(TUNE_MV_LK) == 0 && sliver_shape(bits, R, K, S, sparse_mask != nullptr)) {
+        const bool ok = bits == 3 ? launch_skinny_slivers<3>(a, st) : launch_skinny_slivers<2>(a, st);
+        if (ok) return true;
+    }
+    // more 64-column strips than CUs, fewer than twice as many: one workgroup per CU, the strips' units shared evenly
+    // (16:32 with more than 16 rows has no 64-column strips)
+    if (cw == 4 && tuning(TUNE_NO_BALANCE) == 0 && balanced_shape(R, K, S) && ws.counters != nullptr &&
+        ws.scratch_bytes >= skinny_balanced_part_bytes(S)) {
+        a.counters = reinterpret_cast<int*>(ws.counters);
+        a.part = reinterpret_cast<float*>(ws.scratch);
+        a.units_per_wave = 0;
+        const bool ok = sparse_mask ? launch_skinny_balanced<4, true>(a, st)
+                      : bits == 4 ? launch_skinny_balanced<4, false>(a, st)
+                      : bits == 3 ? launch_skinny_balanced<3, false>(a, st) : launch_skinny_balanced<2, false>(a, st);
+        if (ok) return true;
+        a.counters = nullptr;
+        a.part = nullptr;
+    }
     return launch(cw, waves, 1);
 }
 

@@ -56,8 +56,10 @@ def test_baseline_shape_with_few_rows():
     # the few-row legs that bench.py reports at the BASELINE shape: 2 rows through the matvec kernel (a row per
     # MFMA result register), 8 rows through the few-row kernel, 64 rows through the kernel with shared staging
     assert d("mtx", 4, 1, 2, K, S, 128).startswith("matvec_kernel<bits=4,dense,lane_groups=2,prefetch=0,rows=2> strips=160 splits=4")
-    assert d("mtx", 4, 1, 8, K, S, 128).startswith("skinny_kernel<bits=4,dense,columns_per_lane=4,row_tiles=1> strips=320")
-    assert d("vec", 4, 8, 1, K, S, 128).startswith("skinny_kernel<bits=4,dense,columns_per_lane=4,row_tiles=1> strips=320")
+    # (320 strips of 64 columns on 256 CUs: 256 workgroups share the strips' units evenly)
+    shared = "skinny_kernel<bits=4,dense,columns_per_lane=4,row_tiles=1,balanced> strips=320 row_blocks=1 workgroups=256 waves=8"
+    assert d("mtx", 4, 1, 8, K, S, 128).startswith(shared)
+    assert d("vec", 4, 8, 1, K, S, 128).startswith(shared)
     assert d("mtx", 4, 1, 64, K, S, 128).startswith("wide_rows_kernel<bits=4,dense,row_tiles=4> strips=80 row_blocks=1 ksplit=3")
     # a single row through the matmul entry: the matvec kernel (all formats), the same launch as the matvec entry's
     for bits, sparse, g in ((4, False, 128), (3, False, 128), (2, False, 128), (4, True, 64)):
@@ -107,6 +109,31 @@ def test_every_shape_gets_a_kernel_within_its_limits(fmt):
             bare = d("mtx", bits, 1, rows, k, s, g, sparse, workspace_bytes=0)
             n2, f2, _ = fields(bare)
             assert n2 in KERNELS and f2.get("ksplit", 1) == 1 and f2.get("splits", 1) == 1, bare
+
+
+def evenly_shared(line):
+    return "balanced" in line or "columns_per_lane=4+1" in line
+
+
+def test_more_strips_than_cus_are_shared_out_evenly_within_limits():
+    assert evenly_shared(d("mtx", 4, 1, 8, 12288, 28672, 128)) and evenly_shared(d("mtx", 4, 1, 16, 3072, 16448, 64, True))
+    assert not evenly_shared(d("mtx", 4, 1, 17, 3072, 17408, 128))          # more than 16 rows
+    assert not evenly_shared(d("mtx", 4, 1, 8, 2048, 20480, 128))           # a short K
+    assert not evenly_shared(d("mtx", 4, 1, 8, 8192, 22016, 128))           # many more strips than CUs, K not long
+    assert not evenly_shared(d("mtx", 4, 1, 8, 5120, 16384, 128))           # a strip per CU
+    # without a workspace there is nowhere to sum a shared strip: a workgroup per strip; slivers need none
+    assert not evenly_shared(d("mtx", 4, 1, 8, 5120, 20480, 128, False, 0))
+    assert "columns_per_lane=4+1" in d("mtx", 3, 1, 8, 5120, 20480, 128, False, 0)
+    # tuning key 9 = 1 switches both off
+    capi.tune(9, 1)
+    try:
+        assert not evenly_shared(d("mtx", 4, 1, 8, K, S, 128)) and not evenly_shared(d("mtx", 3, 1, 8, K, S, 128))
+    finally:
+        capi.tune(9, 0)
+    # the shared launch's partial tiles fit the workspace that the size query asks for
+    for bits, sparse in ((4, False), (4, True)):
+        for k, s in ((3072, 16448), (5120, 20480), (12288, 32704)):
+            assert capi.matmul_workspace_bytes(1, 16, k, s, sparse) >= 2 * ((s // 64) * 2 * 8192), (k, s)
 
 
 def test_workspace_sizes_are_consistent():

@@ -550,3 +550,84 @@ def test_more_batch_elements_than_one_launch_takes(H, bits, sparse, B):
     p = O.make_problem(bits=bits, K=1024, S=512, M=1, B=B, group_size=g, sparse=sparse, seed=B, **kw)
     prior = np.random.default_rng(B).standard_normal((B, 1, 512)).astype(np.float16)
     _check(H, p, "vec", prior=prior)
+
+
+# ---- more 64-column strips than CUs, up to 16 rows: the work is shared out evenly over one workgroup per CU.
+# int4 and 16:32: the workgroups share the strips' units (a strip that two of them share is summed through the
+# workspace); int3 and int2 with at most a quarter more strips than CUs: no sharing, a workgroup takes 64 or 80
+# columns.  Tuning key 9 = 1: a workgroup per strip.
+EVEN_SHAPES = [(8, 3072, 16448, 128), (5, 3072, 20480, 64), (16, 3072, 20416, -1), (9, 3200, 17408, 64),
+               (6, 10240, 20544, 128), (2, 4096, 18432, 256)]
+
+
+def _evenly_shared(line):
+    return ("balanced" in line and "workgroups=256" in line) or ("columns_per_lane=4+1" in line and "strips=256" in line)
+
+
+@pytest.mark.parametrize("bits,sparse", [(4, False), (3, False), (2, False), (4, True)])
+@pytest.mark.parametrize("M,K,S,g", EVEN_SHAPES)
+def test_few_rows_evenly_shared_launch(H, bits, sparse, M, K, S, g):
+    capi = H.capi
+    line = capi.describe_launch("mtx", bits, 1, M, K, S, g, sparse)
+    if not line.startswith("matvec_kernel"):             # (two to four rows of a dense format may go to the matvec kernel)
+        assert _evenly_shared(line), line
+        assert ("4+1" in line) == (not sparse and bits != 4 and S <= 20480)
+    p = _problem(bits, K=K, S=S, M=M, group_size=g, seed=M + S, sparse=sparse)
+    d = H.dev_problem(p)
+    exact, f32 = H.oracles(p)
+    ws = capi.new_matmul_workspace(1, M, K, S, sparse)
+    outs = []
+    for _ in range(3):                                   # one workspace: the strips' counters must come back to zero
+        o = torch.full((1, M, S), -5.0, dtype=torch.float16, device="cuda")
+        capi.matmul(bits, o, d["matrix"], d["states"], d["scales"], d["zeros"], g, d["mask"], ws)
+        torch.cuda.synchronize()
+        outs.append(o.cpu().numpy())
+    capi.workspace_status(ws)                            # (raises if a hand-over has failed on it)
+    # (one group over all of K: the sums of the offsets reach 10^6 and more in fp32 -- the floor of 1 x RMS only)
+    H.assert_product_close(outs[0], exact, f32, kind="vec", tight=g > 0 and line.startswith(("skinny_kernel", "matvec_kernel")))
+    assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[0], outs[2])
+    capi.tune(9, 1)                                      # a workgroup per strip
+    try:
+        assert not _evenly_shared(capi.describe_launch("mtx", bits, 1, M, K, S, g, sparse))
+        ref = H.run_capi(p, d, "mtx")
+    finally:
+        capi.tune(9, 0)
+    assert O.max_rel_error(ref.astype(np.float64), outs[0]) < H.TOL_EXACT
+
+
+@pytest.mark.parametrize("bits,sparse", [(4, False), (3, False), (2, False), (4, True)])
+def test_few_rows_evenly_shared_exponent_mode_batches_and_prior_outs(H, bits, sparse):
+    # five batch elements through the matvec entry, which adds onto outs; exponent-mode columns in a strip that two
+    # workgroups share (strip 1 of 320: workgroup 0 takes its first quarter) and in one that a workgroup has to itself
+    K, S, g = 3072, 20480, 128 if not sparse else 64
+    assert _evenly_shared(H.capi.describe_launch("vec", bits, 5, 1, K, S, g, sparse))
+    p = _problem(bits, K=K, S=S, M=1, B=5, group_size=g, seed=12, sparse=sparse)
+    p["scales"][0, 64 + 5] *= np.float16(-1)
+    p["scales"][(K // g) - 1, 64 + 40:64 + 44] *= np.float16(-1)
+    p["scales"][3, 4 * 64 + 17] *= np.float16(-1)
+    prior = np.random.default_rng(2).standard_normal((5, 1, S)).astype(np.float16)
+    _check(H, p, "vec", prior=prior)
+
+
+def test_few_rows_shared_strips_take_turns_on_one_workspace(H):
+    """a matvec, the few-row product with shared strips and a matvec again on one workspace: the strips' counters and
+    partial tiles must not disturb the matvec's hand-over slots, nor the other way round"""
+    capi = H.capi
+    K, S, g = 3072, 20480, 128
+    assert "balanced" in capi.describe_launch("mtx", 4, 1, 8, K, S, g)
+    pv = _problem(4, K=K, S=S, M=1, group_size=g, seed=3)
+    pm = dict(pv, M=8, states=np.random.default_rng(4).standard_normal((1, 8, K)).astype(np.float16))
+    dv, dm = H.dev_problem(pv), H.dev_problem(pm)
+    ws = capi.new_matmul_workspace(1, 8, K, S, False)
+    assert ws.numel() * ws.element_size() >= capi.lib().int4mm_workspace_bytes(S)
+    ev, fv = H.oracles(pv)
+    em, fm = H.oracles(pm)
+    for _ in range(2):
+        ov = torch.zeros((1, 1, S), dtype=torch.float16, device="cuda")
+        capi.matvec(4, ov, dv["matrix"], dv["states"], dv["scales"], dv["zeros"], g, None, ws)
+        om = torch.zeros((1, 8, S), dtype=torch.float16, device="cuda")
+        capi.matmul(4, om, dm["matrix"], dm["states"], dm["scales"], dm["zeros"], g, None, ws)
+        torch.cuda.synchronize()
+        H.assert_product_close(ov.cpu().numpy(), ev, fv, kind="vec")
+        H.assert_product_close(om.cpu().numpy(), em, fm, kind="vec")
+    capi.workspace_status(ws)
