@@ -262,6 +262,15 @@ __host__ __device__ constexpr uint32_t pair_selector(int a, int b) {
 // Staged states per unit: for each block 16 dwords {x_j, x_j+4}, ordered as the
 // dense int4 path.
 
+// EXPO: the exponent quantisation of the same rows.  A kept row's half 0x001q becomes +-2^(q & 7) -- the code's low
+// three bits added to the exponent field of 1.0 (the "kept" flag times 0x3C0 is fp16 1.0), its top bit the sign --
+// and a dropped row's stays 0: accA = sum over kept rows of x * +-2^e, exactly; accM as before.
+__device__ __forceinline__ uint32_t sparse_expo_halves(uint32_t h, uint32_t kept) {
+    const uint32_t t = h << 10;
+    const uint32_t magnitude = __umul24(kept, 0x3C0u) + (t & 0x1C001C00u);
+    return ((t << 2) & 0x80008000u) | magnitude;
+}
+template <bool EXPO = false>
 __device__ __forceinline__ void unit_fast_sparse(const Unit<4, true>& u, const h16* xp, const char* lut,
                                                  f32x4 accA[4], f32x4 accM[4]) {
     const uint32_t NIB = in_vgpr(0x0F0F0F0Fu), FLAG = in_vgpr(0x10101010u), KEPT = in_vgpr(0x00100010u);
@@ -283,14 +292,19 @@ __device__ __forceinline__ void unit_fast_sparse(const Unit<4, true>& u, const h
                 const uint32_t even = and_or(chunk, NIB, FLAG), odd = and_or(chunk >> 4, NIB, FLAG);
                 stream >>= __builtin_popcount(mb4);
                 const u32x4 px = *reinterpret_cast<const u32x4*>(xw + hb * 16 + i * 4);
-                const uint32_t b0 = __builtin_amdgcn_perm(odd, even, sel.x);
-                const uint32_t b1 = __builtin_amdgcn_perm(odd, even, sel.y);
-                const uint32_t b2 = __builtin_amdgcn_perm(odd, even, sel.z);
-                const uint32_t b3 = __builtin_amdgcn_perm(odd, even, sel.w);
+                uint32_t b0 = __builtin_amdgcn_perm(odd, even, sel.x);
+                uint32_t b1 = __builtin_amdgcn_perm(odd, even, sel.y);
+                uint32_t b2 = __builtin_amdgcn_perm(odd, even, sel.z);
+                uint32_t b3 = __builtin_amdgcn_perm(odd, even, sel.w);
+                const uint32_t k0 = b0 & KEPT, k1 = b1 & KEPT, k2 = b2 & KEPT, k3 = b3 & KEPT;
+                if constexpr (EXPO) {
+                    b0 = sparse_expo_halves(b0, k0); b1 = sparse_expo_halves(b1, k1);
+                    b2 = sparse_expo_halves(b2, k2); b3 = sparse_expo_halves(b3, k3);
+                }
                 ra = mma4(px.x, px.y, b0, b1, ra);
-                rm = mma4(px.x, px.y, b0 & KEPT, b1 & KEPT, rm);
+                rm = mma4(px.x, px.y, k0, k1, rm);
                 ra = mma4(px.z, px.w, b2, b3, ra);
-                rm = mma4(px.z, px.w, b2 & KEPT, b3 & KEPT, rm);
+                rm = mma4(px.z, px.w, k2, k3, rm);
             }
             accA[c] = ra;
             accM[c] = rm;
@@ -659,7 +673,7 @@ void matvec_kernel(MatvecArgs a) {
         // exponent-mode columns: a second pass over the units that have any (the group's scales
         // are looked at first; most units are skipped).  Dense formats run the same operands
         // through the exponent decode -- no offsets to remove, y += z * sum(x) - s * sum(x * +-2^e);
-        // 16:32 takes the general decoder.
+        // 16:32 likewise, with the sum over the kept rows from its second accumulator.
         if (__builtin_amdgcn_ballot_w64(need_general) != 0 && work) {
             for (int v = wg_u0 + grp; v < wg_u1; v += ng) {
                 const u32x2 sc2 = *reinterpret_cast<const u32x2*>(a.scales + (int64_t)(v / a.group_units) * a.S + col);
@@ -690,11 +704,13 @@ void matvec_kernel(MatvecArgs a) {
                         }
                     }
                 } else {
-                    if (!(expo[0] | expo[1] | expo[2] | expo[3])) continue;
-                    float acc[4], xsv[4];
-                    unit_generic<BITS, SPARSE>(ua, a.x + v * 64, expo, acc, xsv);
+                    // 16:32: the same expansion of the kept codes, their halves turned into +-2^e; M = 2^20 accM
+                    f32x4 accA[4], accM[4];
 #pragma unroll
-                    for (int c = 0; c < 4; ++c) y[c] += expo[c] ? ze[c] * xsv[c] - sc[c] * acc[c] : 0.f;
+                    for (int c = 0; c < 4; ++c) { accA[c] = f32x4{0.f, 0.f, 0.f, 0.f}; accM[c] = f32x4{0.f, 0.f, 0.f, 0.f}; }
+                    unit_fast_sparse<true>(ua, xs + (v - wg_u0) * (Fmt<BITS, SPARSE>::XS / 2), reinterpret_cast<const char*>(lut), accA, accM);
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) y[c] += expo[c] ? ze[c] * (1048576.f * accM[c][0]) - sc[c] * accA[c][0] : 0.f;
                 }
             }
         }

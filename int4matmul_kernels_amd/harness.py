@@ -13,6 +13,7 @@ are additionally timed with HIP events.
     python -m int4matmul_kernels_amd.harness --quick         # small shapes only
     python -m int4matmul_kernels_amd.harness --config 4,5120,20480,2048,128,0
     python -m int4matmul_kernels_amd.harness --only C3,C3t --clocks 3    # + shader clock under load
+    python -m int4matmul_kernels_amd.harness --only C3,C4m --exponent-every 40   # one group in 40 in exponent mode
 
 A configuration is bits,K,S,M,group,sparse[,B].
 """
@@ -51,10 +52,12 @@ QUICK = [
 ]
 
 
-def make_case(bits, K, S, M, group, sparse, B, seed=0):
+def make_case(bits, K, S, M, group, sparse, B, seed=0, exponent_every=0):
     """Synthetic problem: codes U{0..2^bits-1}, scales U(0.001, 0.02) (int4) or
     U(0.004, 0.08), zeros U(0, 15) for int4 and the mid-code constant otherwise,
-    states N(0, 1); generated on the CPU with a fixed seed, packed on the device."""
+    states N(0, 1); generated on the CPU with a fixed seed, packed on the device.
+    `exponent_every` = n > 0: every n-th group of every column gets a negative scale, which switches
+    that (group, column) to the exponent quantisation (matmul.cuh:414-428)."""
     gen = torch.Generator().manual_seed(seed)
     codes = torch.randint(0, 1 << bits, (K, S), generator=gen, dtype=torch.int32).to(torch.uint8)
     G = 1 if group < 0 else (K + group - 1) // group
@@ -64,6 +67,8 @@ def make_case(bits, K, S, M, group, sparse, B, seed=0):
         zeros = (torch.rand((G, S), generator=gen) * 15.0).half()
     else:
         zeros = torch.full((G, S), ((1 << bits) - 1) / 2.0).half()
+    if exponent_every > 0:
+        scales[exponent_every - 1::exponent_every] *= -1
     states = torch.randn((B, M, K), generator=gen).half()
     codes_d = codes.to(DEV)
     mask = None
@@ -96,6 +101,14 @@ def reference_matrices(c):
     s16, z16 = c["scales"][rows], c["zeros"][rows]
     w16 = (q.half() - z16) * s16                                     # two fp16 roundings
     w32 = (q.float() - z16.float()) * s16.float()
+    expo = s16 < 0
+    if bool(expo.any()):
+        # exponent mode (matmul.cuh:127-136): +-2^(low bits) * (-scale) + zero, rounded once
+        low = (q & ((1 << (c["bits"] - 1)) - 1)).to(torch.int32)
+        iv = torch.where((q >> (c["bits"] - 1)) & 1 == 1, -1.0, 1.0).double() * torch.pow(2.0, low.double())
+        we = iv * (-s16.double()) + z16.double()
+        w16 = torch.where(expo, we.half(), w16)
+        w32 = torch.where(expo, we.float(), w32)
     if c["keep"] is not None:
         w16 = w16 * c["keep"].half()
         w32 = w32 * c["keep"].float()
@@ -248,6 +261,8 @@ def main(argv=None):
     ap.add_argument("--clocks", type=float, default=0.0, metavar="SECONDS",
                     help="also run each case for SECONDS and report the shader clock rocm-smi shows meanwhile")
     ap.add_argument("--only", default="", help="comma-separated names of standard configurations to run")
+    ap.add_argument("--exponent-every", type=int, default=0, metavar="N",
+                    help="every N-th quantisation group of every column in exponent mode (a negative scale)")
     args = ap.parse_args(argv)
     if not torch.cuda.is_available():
         raise SystemExit("the harness needs a GPU")
@@ -263,7 +278,7 @@ def main(argv=None):
     rows = []
     for case in cases:
         name, bits, K, S, M, group, sparse, B = case
-        c = make_case(bits, K, S, M, group, sparse, B)
+        c = make_case(bits, K, S, M, group, sparse, B, exponent_every=args.exponent_every)
         rows.append(run_case(name, c, ext, repeats=args.repeats, cold=args.cold, clocks=args.clocks))
         print("%-5s int%d K=%d S=%d M=%d B=%d g=%d %s: %.2f us, %s, mean rel err %.2e %s%s" % (
             name, bits, K, S, M, B, group, "16:32" if sparse else "dense", rows[-1]["quant_event_us"],

@@ -83,6 +83,24 @@ def test_matvec_exponent_mode_columns(H, bits, sparse):
         H.assert_product_close(got, exact, f32, kind="vec" if kind == "vec" else H.matmul_kind(p))
 
 
+@pytest.mark.parametrize("bits,sparse", FORMATS)
+def test_matvec_exponent_mode_groups_split_k(H, bits, sparse):
+    """K = 8192 split over several workgroups, 64-row groups: exponent mode in whole groups, in every third column of
+    another and in single (group, column) pairs -- the second pass over the units that hold any, for 16:32 with the
+    kept codes expanded as in the first pass and their halves turned into +-2^e"""
+    K, S, g = 8192, 2048, 64
+    p = _problem(bits, sparse, K=K, S=S, M=1, group_size=g, seed=11)
+    assert "splits=" in H.capi.describe_launch("vec", bits, 1, 1, K, S, g, sparse)
+    sc = p["scales"]
+    sc[5] *= np.float16(-1)
+    sc[77, ::3] *= np.float16(-1)
+    sc[np.arange(128), np.arange(128) * 37 % S] *= np.float16(-1)
+    exact, f32 = H.oracles(p)
+    prior = np.random.default_rng(3).standard_normal((1, 1, S)).astype(np.float16)
+    got = H.run_capi(p, H.dev_problem(p), "vec", outs_init=prior)
+    H.assert_product_close(got, exact, f32, prior=prior)
+
+
 @pytest.mark.parametrize("bits,sparse,K", [(4, False, 5120), (3, False, 1024), (2, False, 2048),
                                            (4, True, 16384)])
 def test_degenerate_known_answer(H, bits, sparse, K):
