@@ -46,6 +46,9 @@
 
 namespace i4 {
 
+// magic numbers (div_magic) of the divisors of the balanced launch's range arithmetic: K / 64, the group's units, q, q + 1
+struct BalancedMagics { uint32_t units, group_units, share_lo, share_hi; };
+
 struct SkinnyArgs {
     h16* outs;
     const uint32_t* matrix;
@@ -67,6 +70,7 @@ struct SkinnyArgs {
     // balanced launch of the few-row kernel (more strips than CUs): `bal_wgs` workgroups share the strips' units
     // evenly, workgroup i takes [i q + i r / wgs, (i + 1) q + (i + 1) r / wgs) of strips x units, strip-major
     int bal_wgs, bal_q, bal_r;
+    BalancedMagics bal_magics;
     // launch with a fifth column per lane: the first `wide_wgs` workgroups take 80 columns, the others 64
     int wide_wgs;
 };
@@ -188,8 +192,17 @@ __device__ __forceinline__ h16x8 exact_operand(uint32_t f, uint32_t m0, uint32_t
 // and number of waves; for the workgroup's copy of scales and zeros in LDS: the first group of each segment
 // and where each segment's groups start (goff3: all groups).
 struct BalancedShare { int strip0, mine, lo, hi, wave0, waves, glo0, glo1, glo2, goff1, goff2, goff3; };
-// a / b for 0 <= a < 2^22, b >= 1 through the float reciprocal (one step of correction either way): a dozen such
-// quotients stand between a wave's start and its first loads, and the compiler's exact division is ~35 instructions
+// a / b for 0 <= a < 2^22, b >= 1 with b's magic number floor(2^32 / b) + 1 (2^32 - 1 for b = 1): the high word of
+// the product is the quotient or one off, in integer scalar instructions -- a dozen such quotients stand between a
+// wave's start and its first loads, and the compiler's exact division is ~35 vector instructions each
+__host__ __device__ inline uint32_t div_magic(uint32_t b) { return b <= 1 ? 0xFFFFFFFFu : (uint32_t)(0x100000000ull / b) + 1u; }
+__host__ __device__ inline int magic_div(int a, int b, uint32_t magic) {
+    int q = (int)(uint32_t)(((uint64_t)(uint32_t)a * magic) >> 32);
+    if (q * b > a) --q;
+    if ((q + 1) * b <= a) ++q;
+    return q;
+}
+// (the same through the float reciprocal, for a divisor without a magic number at hand)
 __device__ __forceinline__ int small_div(int a, int b, float inv_b) {
     int q = (int)((float)a * inv_b);
     int r = a - q * b;
@@ -197,14 +210,15 @@ __device__ __forceinline__ int small_div(int a, int b, float inv_b) {
     if (r >= b) ++q;
     return q;
 }
-__device__ __forceinline__ BalancedShare balanced_share(int q, int r, int i, int units, int group_units, int nwaves, int wave) {
+__device__ __forceinline__ BalancedShare balanced_share(int q, int r, const BalancedMagics& mg, int i, int units, int group_units,
+                                                        int nwaves, int wave) {
     BalancedShare b{};
     constexpr int WGS = 256;                                         // (SK_BAL_WGS, the host side's constant)
     const int lo = i * q + ((i * r) >> 8), hi = (i + 1) * q + (((i + 1) * r) >> 8);
     const int share = hi - lo;
     static_assert(WGS == 1 << 8, "the shifts above");
-    const float inv_units = 1.f / (float)units, inv_gu = 1.f / (float)group_units, inv_share = 1.f / (float)share;
-    b.strip0 = small_div(lo, units, inv_units);
+    const uint32_t share_magic = share == q ? mg.share_lo : mg.share_hi;
+    b.strip0 = magic_div(lo, units, mg.units);
     int seg_lo[3], seg_n[3], seg_w[3], dealt = 0;
 #pragma unroll
     for (int k = 0; k < 3; ++k) {
@@ -212,7 +226,7 @@ __device__ __forceinline__ BalancedShare balanced_share(int q, int r, int i, int
         const int from = max(lo, s0), to = min(hi, s0 + units);
         seg_lo[k] = from - s0;
         seg_n[k] = max(0, to - from);
-        seg_w[k] = seg_n[k] > 0 ? max(1, small_div(seg_n[k] * nwaves + share / 2, share, inv_share)) : 0;
+        seg_w[k] = seg_n[k] > 0 ? max(1, magic_div(seg_n[k] * nwaves + share / 2, share, share_magic)) : 0;
         dealt += seg_w[k];
     }
     // the rounding may deal a wave or two too many or too few: take from the segment with the fewest units per
@@ -243,12 +257,12 @@ __device__ __forceinline__ BalancedShare balanced_share(int q, int r, int i, int
         if (wave >= w0 && wave < w0 + seg_w[k]) { b.mine = k; b.wave0 = w0; b.waves = seg_w[k]; b.lo = seg_lo[k]; b.hi = seg_lo[k] + seg_n[k]; }
         w0 += seg_w[k];
     }
-    const int g0 = small_div(seg_lo[0], group_units, inv_gu), g1 = small_div(seg_lo[1], group_units, inv_gu),
-              g2 = small_div(seg_lo[2], group_units, inv_gu);
+    const int g0 = magic_div(seg_lo[0], group_units, mg.group_units), g1 = magic_div(seg_lo[1], group_units, mg.group_units),
+              g2 = magic_div(seg_lo[2], group_units, mg.group_units);
     b.glo0 = g0; b.glo1 = g1; b.glo2 = g2;
-    b.goff1 = seg_n[0] > 0 ? small_div(seg_lo[0] + seg_n[0] - 1, group_units, inv_gu) + 1 - g0 : 0;
-    b.goff2 = b.goff1 + (seg_n[1] > 0 ? small_div(seg_lo[1] + seg_n[1] - 1, group_units, inv_gu) + 1 - g1 : 0);
-    b.goff3 = b.goff2 + (seg_n[2] > 0 ? small_div(seg_lo[2] + seg_n[2] - 1, group_units, inv_gu) + 1 - g2 : 0);
+    b.goff1 = seg_n[0] > 0 ? magic_div(seg_lo[0] + seg_n[0] - 1, group_units, mg.group_units) + 1 - g0 : 0;
+    b.goff2 = b.goff1 + (seg_n[1] > 0 ? magic_div(seg_lo[1] + seg_n[1] - 1, group_units, mg.group_units) + 1 - g1 : 0);
+    b.goff3 = b.goff2 + (seg_n[2] > 0 ? magic_div(seg_lo[2] + seg_n[2] - 1, group_units, mg.group_units) + 1 - g2 : 0);
     return b;
 }
 
@@ -279,7 +293,7 @@ __global__ __launch_bounds__(512) void skinny_kernel(SkinnyArgs a) {
     int seg_wave0 = 0, seg_waves = nwaves;                      // the waves that work on the same strip
     BalancedShare bs{};
     if constexpr (BAL) {
-        bs = balanced_share(a.bal_q, a.bal_r, blockIdx.x, units, a.group_units, nwaves, wave);
+        bs = balanced_share(a.bal_q, a.bal_r, a.bal_magics, blockIdx.x, units, a.group_units, nwaves, wave);
         strip = bs.strip0 + bs.mine;
         split_lo = bs.lo;
         split_hi = bs.hi;
@@ -1297,6 +1311,7 @@ static bool launch_skinny_balanced(SkinnyArgs a, hipStream_t st) {
     a.bal_wgs = SK_BAL_WGS;
     a.bal_q = (int)(total / SK_BAL_WGS);
     a.bal_r = (int)(total % SK_BAL_WGS);
+    a.bal_magics = {div_magic((uint32_t)units), div_magic((uint32_t)a.group_units), div_magic((uint32_t)a.bal_q), div_magic((uint32_t)a.bal_q + 1u)};
     // scales in LDS: a workgroup's range is less than two strips long and touches at most three
     const int groups = 2 * ((units + a.group_units - 1) / a.group_units) + 3;
     size_t lds = (size_t)WAVES * SK_WAVE_LDS + 16 + (size_t)groups * 16 * CW * 4;
