@@ -29,6 +29,9 @@ HIP_FLAGS = [
     "-fgpu-rdc" if False else "-fno-gpu-rdc",
     # packed-FP32 VALU ops are switched off for every device compile
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # the first dwords of a kernel's explicit arguments arrive in registers with the wave (scalar leading arguments
+    # only: a record passed by value is still fetched by the wave itself)
+    "-mllvm", "-amdgpu-kernarg-preload-count=12",
     "-Wall", "-Wno-unused-function", "-Wno-unknown-warning-option", "-Wno-unused-command-line-argument",
 ]
 

@@ -411,7 +411,12 @@ __device__ __forceinline__ uint64_t slot_load(const uint64_t* p) {
 // reduction area and the hand-over slots (slot row = split * NR + row) are kept per row.
 template <int BITS, bool SPARSE, int LK, bool PF, int NR = 1>
 __global__ __launch_bounds__(MV_MAX_WAVES * WAVE)
-void matvec_kernel(MatvecArgs a) {
+void matvec_kernel(const uint32_t* pre_matrix, const h16* pre_scales, const h16* pre_zeros, const h16* pre_x, int pre_S,
+                   int pre_units_per_wg, int pre_group_units, int pre_units_total, MatvecArgs a) {
+    // (the arguments that the first loads depend on, once more in front of the record: the first dwords of a kernel's
+    // arguments can be handed to a wave in registers at its start, a record's fields are fetched by the wave itself)
+    a.matrix = pre_matrix; a.scales = pre_scales; a.zeros = pre_zeros; a.x = pre_x; a.S = pre_S;
+    a.units_per_wg = pre_units_per_wg; a.group_units = pre_group_units; a.units_total = pre_units_total;
     constexpr bool FAST = Fmt<BITS, SPARSE>::FAST;
     static_assert(NR == 1 || ((NR == 2 || NR == 4) && FAST && !SPARSE), "several rows: dense formats only");
     constexpr int LC = WAVE / LK;                 // column lanes per lane group
@@ -855,7 +860,7 @@ static size_t matvec_lds_bytes(int units_per_wg, int threads, int nr) {
 template <int BITS, int NR>
 static void launch_rows(const MatvecArgs& a, int lk, bool pf, dim3 grid, dim3 block, hipStream_t st) {
     const size_t lds = matvec_lds_bytes<BITS, false>(a.units_per_wg, (int)block.x, NR);
-#define I4_LAUNCH(LK_, PF_) hipLaunchKernelGGL((matvec_kernel<BITS, false, LK_, PF_, NR>), grid, block, lds, st, a)
+#define I4_LAUNCH(LK_, PF_) hipLaunchKernelGGL((matvec_kernel<BITS, false, LK_, PF_, NR>), grid, block, lds, st, a.matrix, a.scales, a.zeros, a.x, a.S, a.units_per_wg, a.group_units, a.units_total, a)
     if (lk == 1) { if (pf) I4_LAUNCH(1, true); else I4_LAUNCH(1, false); }
     else if (lk == 2) { if (pf) I4_LAUNCH(2, true); else I4_LAUNCH(2, false); }
     else { if (pf) I4_LAUNCH(4, true); else I4_LAUNCH(4, false); }
@@ -865,7 +870,7 @@ static void launch_rows(const MatvecArgs& a, int lk, bool pf, dim3 grid, dim3 bl
 template <int BITS, bool SPARSE>
 static void launch(const MatvecArgs& a, int lk, bool pf, dim3 grid, dim3 block, hipStream_t st) {
     const size_t lds = matvec_lds_bytes<BITS, SPARSE>(a.units_per_wg, (int)block.x, 1);
-#define I4_LAUNCH(LK_, PF_) hipLaunchKernelGGL((matvec_kernel<BITS, SPARSE, LK_, PF_>), grid, block, lds, st, a)
+#define I4_LAUNCH(LK_, PF_) hipLaunchKernelGGL((matvec_kernel<BITS, SPARSE, LK_, PF_>), grid, block, lds, st, a.matrix, a.scales, a.zeros, a.x, a.S, a.units_per_wg, a.group_units, a.units_total, a)
     if (lk == 1) { if (pf) I4_LAUNCH(1, true); else I4_LAUNCH(1, false); }
     else if (lk == 2) { if (pf) I4_LAUNCH(2, true); else I4_LAUNCH(2, false); }
     else { if (pf) I4_LAUNCH(4, true); else I4_LAUNCH(4, false); }

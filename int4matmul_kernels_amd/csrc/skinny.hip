@@ -274,7 +274,12 @@ __device__ __forceinline__ BalancedShare balanced_share(int q, int r, const Bala
 // XC = 1: a fifth column per lane (CW = 4 only, dense formats): the workgroup's columns are four or five slivers of
 // 16, the lane's four adjacent columns in the first four and column j of the fifth (a.wide_wgs workgroups have one)
 template <int BITS, int CW, int RT, bool SPARSE, bool BAL = false, int XC = 0>
-__global__ __launch_bounds__(512) void skinny_kernel(SkinnyArgs a) {
+__global__ __launch_bounds__(512) void skinny_kernel(const uint32_t* pre_matrix, const h16* pre_x, const h16* pre_scales, const h16* pre_zeros,
+                                                   int pre_S, int pre_K, int pre_group_units, int pre_units, SkinnyArgs a) {
+    // (what the first loads depend on, once more in front of the record: the first dwords of a kernel's arguments
+    // reach a wave in registers at its start, a record's fields are fetched by the wave itself)
+    a.matrix = pre_matrix; a.x = pre_x; a.scales = pre_scales; a.zeros = pre_zeros; a.S = pre_S; a.K = pre_K;
+    a.group_units = pre_group_units; a.units_per_wave = pre_units;
     using F = SkFmt<BITS, SPARSE>;
     constexpr int NL = F::LOADS;
     constexpr int PF = (BITS == 3 && CW == 4) || (SPARSE && CW == 4) ? 2 : 4, MT = RT == 4 ? 2 : 1;
@@ -769,7 +774,12 @@ __global__ __launch_bounds__(512) void skinny_kernel(SkinnyArgs a) {
 // per pair of weights on top of the magic-number decode, and the accumulators hold the product itself.
 // K is split across workgroups (blockIdx.z) with the hand-over above, one counter per wave.
 template <int BITS, int MT, bool SPARSE = false>
-__global__ __launch_bounds__(512) void wide_rows_kernel(SkinnyArgs a) {
+__global__ __launch_bounds__(512) void wide_rows_kernel(const uint32_t* pre_matrix, const h16* pre_x, const h16* pre_scales, const h16* pre_zeros,
+                                                   int pre_S, int pre_K, int pre_group_units, int pre_units, SkinnyArgs a) {
+    // (what the first loads depend on, once more in front of the record: the first dwords of a kernel's arguments
+    // reach a wave in registers at its start, a record's fields are fetched by the wave itself)
+    a.matrix = pre_matrix; a.x = pre_x; a.scales = pre_scales; a.zeros = pre_zeros; a.S = pre_S; a.K = pre_K;
+    a.group_units = pre_group_units; a.units_per_split = pre_units;
     using F = SkFmt<BITS, SPARSE>;
     // (units of weights in flight per wave: four; two in the tall 16:32 blocks, whose registers are short)
     constexpr int CW = 2, NL = F::LOADS, PF = (SPARSE && MT > 4) ? 2 : 4, ROWS = 16 * MT, STRIP = 16 * CW, WSTRIP = 8 * STRIP;
@@ -1244,7 +1254,7 @@ static bool launch_wide(SkinnyArgs a, const WidePlan& p, hipStream_t st) {
             hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
             done[slot].fetch_or(bit, std::memory_order_relaxed);
         }
-        hipLaunchKernelGGL(kernel, grid, block, lds, st, a);
+        hipLaunchKernelGGL(kernel, grid, block, lds, st, a.matrix, a.x, a.scales, a.zeros, a.S, a.K, a.group_units, a.units_per_split, a);
     };
     if (p.mt == 1) go(wide_rows_kernel<BITS, 1, SPARSE>, 0);
     else if (p.mt == 2) go(wide_rows_kernel<BITS, 2, SPARSE>, 1);
@@ -1280,7 +1290,7 @@ static bool launch_skinny(const SkinnyArgs& a, int waves, int ksplit, hipStream_
                                 150 * 1024);
             done[slot].fetch_or(bit, std::memory_order_relaxed);
         }
-        hipLaunchKernelGGL(kernel, grid, block, lds, st, a);
+        hipLaunchKernelGGL(kernel, grid, block, lds, st, a.matrix, a.x, a.scales, a.zeros, a.S, a.K, a.group_units, a.units_per_wave, a);
     };
     if (rt <= 1) go(skinny_kernel<BITS, CW, 1, SPARSE>, 0);
     else if (rt <= 2) go(skinny_kernel<BITS, CW, 2, SPARSE>, 1);
@@ -1332,7 +1342,7 @@ static bool launch_skinny_balanced(SkinnyArgs a, hipStream_t st) {
                                 150 * 1024);
             done.fetch_or(bit, std::memory_order_relaxed);
         }
-        hipLaunchKernelGGL(kernel, grid, block, lds, st, a);
+        hipLaunchKernelGGL(kernel, grid, block, lds, st, a.matrix, a.x, a.scales, a.zeros, a.S, a.K, a.group_units, a.units_per_wave, a);
     };
     if (rt <= 1) go(skinny_kernel<BITS, CW, 1, SPARSE, true>);
     else go(skinny_kernel<BITS, CW, 2, SPARSE, true>);            // (up to 16 rows: balanced_shape)
@@ -1376,7 +1386,7 @@ static bool launch_skinny_slivers(SkinnyArgs a, hipStream_t st) {
                                 150 * 1024);
             done.fetch_or(bit, std::memory_order_relaxed);
         }
-        hipLaunchKernelGGL(kernel, grid, block, lds, st, a);
+        hipLaunchKernelGGL(kernel, grid, block, lds, st, a.matrix, a.x, a.scales, a.zeros, a.S, a.K, a.group_units, a.units_per_wave, a);
     };
     if (rt <= 1) go(skinny_kernel<BITS, CW, 1, false, false, 1>);
     else go(skinny_kernel<BITS, CW, 2, false, false, 1>);
