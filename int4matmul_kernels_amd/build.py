@@ -31,7 +31,7 @@ HIP_FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     # the first dwords of a kernel's explicit arguments arrive in registers with the wave (scalar leading arguments
     # only: a record passed by value is still fetched by the wave itself)
-    "-mllvm", "-amdgpu-kernarg-preload-count=12",
+    "-mllvm", "-amdgpu-kernarg-preload-count=16",
     "-Wall", "-Wno-unused-function", "-Wno-unknown-warning-option", "-Wno-unused-command-line-argument",
 ]
 

@@ -65,6 +65,17 @@ __device__ __forceinline__ uint32_t in_vgpr(uint32_t literal) {
     return r;
 }
 
+// a / b for 0 <= a < 2^22, b >= 1 with b's magic number floor(2^32 / b) + 1 (2^32 - 1 for b = 1), which the host passes:
+// the high word of the product is the quotient or one off -- eight integer instructions where the compiler's exact
+// division by a run-time divisor takes ~35
+__host__ __device__ inline uint32_t div_magic(uint32_t b) { return b <= 1 ? 0xFFFFFFFFu : (uint32_t)(0x100000000ull / b) + 1u; }
+__host__ __device__ inline int magic_div(int a, int b, uint32_t magic) {
+    int q = (int)(uint32_t)(((uint64_t)(uint32_t)a * magic) >> 32);
+    if (q * b > a) --q;
+    if ((q + 1) * b <= a) ++q;
+    return q;
+}
+
 // ---- one code -> fp16 weight, the two roundings of the linear mode and the
 // single-rounded fused multiply-add of the exponent mode.
 template <int BITS>

@@ -52,6 +52,7 @@ struct MatvecArgs {
     int units_total;        // K / 64
     int units_per_wg;
     int group_units;        // group size in units (>= 1); huge for a single group
+    uint32_t group_magic;   // div_magic(group_units)
     int splits;             // == gridDim.y
     uint32_t* sticky;       // hand-over error word of the workspace (non-zero: poisoned)
     int spin_limit;         // polls before a reader gives up
@@ -80,7 +81,7 @@ __device__ __forceinline__ void load_unit(Unit<BITS, SPARSE>& u, const MatvecArg
     const int64_t S = a.S;
     // scale / zero first: loads return in order, so the unit is complete when its last weight
     // row arrives instead of two small requests to other pages later
-    const int64_t gofs = (int64_t)(unit / a.group_units) * S + col;
+    const int64_t gofs = (int64_t)magic_div(unit, a.group_units, a.group_magic) * S + col;
     u.sc = *reinterpret_cast<const u32x2*>(a.scales + gofs);
     u.ze = *reinterpret_cast<const u32x2*>(a.zeros + gofs);
     __builtin_amdgcn_sched_barrier(0);
@@ -412,11 +413,11 @@ __device__ __forceinline__ uint64_t slot_load(const uint64_t* p) {
 template <int BITS, bool SPARSE, int LK, bool PF, int NR = 1>
 __global__ __launch_bounds__(MV_MAX_WAVES * WAVE)
 void matvec_kernel(const uint32_t* pre_matrix, const h16* pre_scales, const h16* pre_zeros, const h16* pre_x, int pre_S,
-                   int pre_units_per_wg, int pre_group_units, int pre_units_total, MatvecArgs a) {
+                   int pre_units_per_wg, int pre_group_units, int pre_units_total, uint32_t pre_group_magic, MatvecArgs a) {
     // (the arguments that the first loads depend on, once more in front of the record: the first dwords of a kernel's
     // arguments can be handed to a wave in registers at its start, a record's fields are fetched by the wave itself)
     a.matrix = pre_matrix; a.scales = pre_scales; a.zeros = pre_zeros; a.x = pre_x; a.S = pre_S;
-    a.units_per_wg = pre_units_per_wg; a.group_units = pre_group_units; a.units_total = pre_units_total;
+    a.units_per_wg = pre_units_per_wg; a.group_units = pre_group_units; a.units_total = pre_units_total; a.group_magic = pre_group_magic;
     constexpr bool FAST = Fmt<BITS, SPARSE>::FAST;
     static_assert(NR == 1 || ((NR == 2 || NR == 4) && FAST && !SPARSE), "several rows: dense formats only");
     constexpr int LC = WAVE / LK;                 // column lanes per lane group
@@ -681,7 +682,7 @@ void matvec_kernel(const uint32_t* pre_matrix, const h16* pre_scales, const h16*
         // 16:32 likewise, with the sum over the kept rows from its second accumulator.
         if (__builtin_amdgcn_ballot_w64(need_general) != 0 && work) {
             for (int v = wg_u0 + grp; v < wg_u1; v += ng) {
-                const u32x2 sc2 = *reinterpret_cast<const u32x2*>(a.scales + (int64_t)(v / a.group_units) * a.S + col);
+                const u32x2 sc2 = *reinterpret_cast<const u32x2*>(a.scales + (int64_t)magic_div(v, a.group_units, a.group_magic) * a.S + col);
                 const h16x2 s01 = as_h2(sc2.x), s23 = as_h2(sc2.y);
                 const bool any = !(s01.x >= (h16)0.f) | !(s01.y >= (h16)0.f) | !(s23.x >= (h16)0.f) | !(s23.y >= (h16)0.f);
                 if (__builtin_amdgcn_ballot_w64(any) == 0) continue;
@@ -860,7 +861,7 @@ static size_t matvec_lds_bytes(int units_per_wg, int threads, int nr) {
 template <int BITS, int NR>
 static void launch_rows(const MatvecArgs& a, int lk, bool pf, dim3 grid, dim3 block, hipStream_t st) {
     const size_t lds = matvec_lds_bytes<BITS, false>(a.units_per_wg, (int)block.x, NR);
-#define I4_LAUNCH(LK_, PF_) hipLaunchKernelGGL((matvec_kernel<BITS, false, LK_, PF_, NR>), grid, block, lds, st, a.matrix, a.scales, a.zeros, a.x, a.S, a.units_per_wg, a.group_units, a.units_total, a)
+#define I4_LAUNCH(LK_, PF_) hipLaunchKernelGGL((matvec_kernel<BITS, false, LK_, PF_, NR>), grid, block, lds, st, a.matrix, a.scales, a.zeros, a.x, a.S, a.units_per_wg, a.group_units, a.units_total, a.group_magic, a)
     if (lk == 1) { if (pf) I4_LAUNCH(1, true); else I4_LAUNCH(1, false); }
     else if (lk == 2) { if (pf) I4_LAUNCH(2, true); else I4_LAUNCH(2, false); }
     else { if (pf) I4_LAUNCH(4, true); else I4_LAUNCH(4, false); }
@@ -870,7 +871,7 @@ static void launch_rows(const MatvecArgs& a, int lk, bool pf, dim3 grid, dim3 bl
 template <int BITS, bool SPARSE>
 static void launch(const MatvecArgs& a, int lk, bool pf, dim3 grid, dim3 block, hipStream_t st) {
     const size_t lds = matvec_lds_bytes<BITS, SPARSE>(a.units_per_wg, (int)block.x, 1);
-#define I4_LAUNCH(LK_, PF_) hipLaunchKernelGGL((matvec_kernel<BITS, SPARSE, LK_, PF_>), grid, block, lds, st, a.matrix, a.scales, a.zeros, a.x, a.S, a.units_per_wg, a.group_units, a.units_total, a)
+#define I4_LAUNCH(LK_, PF_) hipLaunchKernelGGL((matvec_kernel<BITS, SPARSE, LK_, PF_>), grid, block, lds, st, a.matrix, a.scales, a.zeros, a.x, a.S, a.units_per_wg, a.group_units, a.units_total, a.group_magic, a)
     if (lk == 1) { if (pf) I4_LAUNCH(1, true); else I4_LAUNCH(1, false); }
     else if (lk == 2) { if (pf) I4_LAUNCH(2, true); else I4_LAUNCH(2, false); }
     else { if (pf) I4_LAUNCH(4, true); else I4_LAUNCH(4, false); }
@@ -982,6 +983,7 @@ bool i4::matvec_rows(int bits, h16* outs, const uint32_t* matrix, const h16* x, 
     a.units_total = units_total;
     a.units_per_wg = ms.upwg;
     a.group_units = (int)(group_size / 64 > 0x7FFFFFF ? 0x7FFFFFF : group_size / 64);
+    a.group_magic = div_magic((uint32_t)a.group_units);
     a.splits = ms.splits;
     a.sticky = ms.splits > 1 ? reinterpret_cast<uint32_t*>(ws.counters - 8) : nullptr;
     a.spin_limit = tuning(TUNE_MV_SPIN) > 0 ? (int)tuning(TUNE_MV_SPIN) : MV_SPIN_LIMIT;
@@ -1103,6 +1105,7 @@ static int matvec_plain(int bits, void* outs, const void* matrix, const void* mu
         a.units_total = units_total;
         a.units_per_wg = upwg;
         a.group_units = (int)gu;
+        a.group_magic = div_magic((uint32_t)a.group_units);
         a.splits = splits;
         a.sticky = splits > 1 ? reinterpret_cast<uint32_t*>(workspace_parts(workspace, workspace_bytes).counters - 8) : nullptr;
         a.spin_limit = tuning(TUNE_MV_SPIN) > 0 ? (int)tuning(TUNE_MV_SPIN) : MV_SPIN_LIMIT;

@@ -192,16 +192,7 @@ __device__ __forceinline__ h16x8 exact_operand(uint32_t f, uint32_t m0, uint32_t
 // and number of waves; for the workgroup's copy of scales and zeros in LDS: the first group of each segment
 // and where each segment's groups start (goff3: all groups).
 struct BalancedShare { int strip0, mine, lo, hi, wave0, waves, glo0, glo1, glo2, goff1, goff2, goff3; };
-// a / b for 0 <= a < 2^22, b >= 1 with b's magic number floor(2^32 / b) + 1 (2^32 - 1 for b = 1): the high word of
-// the product is the quotient or one off, in integer scalar instructions -- a dozen such quotients stand between a
-// wave's start and its first loads, and the compiler's exact division is ~35 vector instructions each
-__host__ __device__ inline uint32_t div_magic(uint32_t b) { return b <= 1 ? 0xFFFFFFFFu : (uint32_t)(0x100000000ull / b) + 1u; }
-__host__ __device__ inline int magic_div(int a, int b, uint32_t magic) {
-    int q = (int)(uint32_t)(((uint64_t)(uint32_t)a * magic) >> 32);
-    if (q * b > a) --q;
-    if ((q + 1) * b <= a) ++q;
-    return q;
-}
+// (a dozen quotients stand between a wave's start and its first loads: magic_div, csrc/common.h)
 // (the same through the float reciprocal, for a divisor without a magic number at hand)
 __device__ __forceinline__ int small_div(int a, int b, float inv_b) {
     int q = (int)((float)a * inv_b);
