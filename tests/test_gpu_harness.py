@@ -25,3 +25,14 @@ def test_harness_full_size_row_per_format():
     assert [r["name"] for r in rows] == names
     for r in rows:
         assert r["ok"] and r["err_quant"] < 1e-2, r            # (mean relative error; the gate itself is 0.1)
+
+
+def test_harness_with_exponent_mode_groups():
+    """every second group of every column in exponent mode: the harness's own truth (from the unpacked codes, in
+    plain torch arithmetic) holds every format's kernels to the same gate"""
+    from int4matmul_kernels_amd import harness
+
+    rows = harness.main(["--quick", "--repeats", "2", "--exponent-every", "2"])
+    assert len(rows) == len(harness.QUICK)
+    for r in rows:
+        assert r["ok"] and r["err_quant"] < 1e-2, r
