@@ -283,20 +283,11 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64, 2) void matmul_kernel(M
 //    stream never drains while waves wait for each other.
 // The steady-state loop body has no branches; a tile that contains exponent-mode
 // groups takes a second pipelined loop whose decode serves either mode (dense formats, 256-column
-// tiles) or a plain loop with the general decode (the others).
+// tiles) or a plain two-stage loop with that decode (the others).
 constexpr int PK = 32;            // K per step of the pipelined kernel
 
-// One 16-byte chunk = 8 consecutive k of one column.  `bits` holds its 8 codes,
-// LSB first, BITS bits apart (bits above 8 * BITS are ignored).
-template <int BITS>
-__device__ __forceinline__ h16x8 dequant_chunk_generic(uint32_t bits, h16 sc, h16 ze) {
-    h16x8 r;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) r[e] = dequant_code<BITS>((bits >> (BITS * e)) & ((1u << BITS) - 1u), sc, ze);
-    return r;
-}
-
-// Linear-mode fast decode of such a chunk, bit-exact.  The two codes of a pair
+// One 16-byte chunk = 8 consecutive k of one column; `bits` holds its 8 codes, LSB first, BITS bits apart (bits
+// above 8 * BITS are ignored).  Linear-mode fast decode of such a chunk, bit-exact.  The two codes of a pair
 // are brought to the low bits of the two halves of a register; mask-and-OR with
 // a magic exponent turns them into {2^a + q_even, 2^b + q_odd}, whose offsets
 // are then subtracted exactly before the reference's two roundings.
@@ -415,16 +406,30 @@ __device__ __forceinline__ h16x8 dequant_chunk_sparse_fast(uint32_t v, uint32_t 
     return bitcast<h16x8>(r);
 }
 
-__device__ __forceinline__ h16x8 dequant_chunk_sparse_generic(uint32_t v, uint32_t m8, h16 sc, h16 ze) {
-    h16x8 r;
+// Either mode per thread without a branch (see dequant_chunk_mixed): the rows' codes ride on 1024 in both halves of
+// a pair, so the packed multiply that moves them to bits 10.. is by 1024 for both.
+__device__ __forceinline__ h16x8 dequant_chunk_sparse_mixed(uint32_t v, uint32_t m8, const uint32_t* lut, bool expo,
+                                                            h16x2 negz, h16x2 s2) {
+    const u32x4 keep = *reinterpret_cast<const u32x4*>(lut + m8 * 8);
+    const u32x2 sel = *reinterpret_cast<const u32x2*>(lut + m8 * 8 + 4);
+    const uint32_t even = v & 0x0F0F0F0Fu, odd = (v >> 4) & 0x0F0F0F0Fu;
+    const uint32_t c03 = __builtin_amdgcn_perm(odd, even, sel.x);
+    const uint32_t c47 = __builtin_amdgcn_perm(odd, even, sel.y);
+    const uint32_t MAGIC = 0x64006400u;
+    const uint32_t h[4] = {__builtin_amdgcn_perm(c03, MAGIC, 0x01050104u), __builtin_amdgcn_perm(c03, MAGIC, 0x01070106u),
+                           __builtin_amdgcn_perm(c47, MAGIC, 0x01050104u), __builtin_amdgcn_perm(c47, MAGIC, 0x01070106u)};
+    const h16x2 unmagic = {(h16)-1024.0f, (h16)-1024.0f}, minus0 = as_h2(0x80008000u);
+    const h16x2 N = expo ? minus0 : negz, B = expo ? -s2 : s2, C = expo ? -negz : minus0;
+    u32x4 r;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-        const bool kept = (m8 >> e) & 1u;
-        r[e] = kept ? dequant_code<4>(v & 15u, sc, ze) : (h16)0.0f;
-        v >>= kept ? 4 : 0;
+    for (int i = 0; i < 4; ++i) {
+        const h16x2 q = as_h2(h[i]) + unmagic;             // exact
+        const h16x2 P = expo ? as_h2(expo_operand<4>(h[i], off2(1024u, 1024u))) : q;
+        r[i] = as_u32(__builtin_elementwise_fma(P + N, B, C)) & keep[i];      // dropped rows -> +0
     }
-    return r;
+    return bitcast<h16x8>(r);
 }
+
 
 // Per-format constants of the pipelined kernel: packed rows per 32-row block and
 // the number of packed words a thread loads per K step for its two chunks.
@@ -562,18 +567,6 @@ __device__ __forceinline__ void pipe_tile(const MatmulArgs& a, const int m0, con
         }
         *reinterpret_cast<h16x8*>(&Bs[stage * B_STAGE + ((bhb * 2 + q) * BN + bn) * 8]) = w;
     };
-    auto write_b_general = [&](const Stage& s, int stage, int q) {
-        h16x8 w;
-        if constexpr (SPARSE) {
-            uint32_t v, m8;
-            sparse_chunk(s, q, v, m8);
-            w = dequant_chunk_sparse_generic(v, m8, stage_scale(s).x, -stage_negzero(s).x);
-        } else {
-            w = dequant_chunk_generic<BITS>(chunk_bits(s, q), stage_scale(s).x, -stage_negzero(s).x);
-        }
-        *reinterpret_cast<h16x8*>(&Bs[stage * B_STAGE + ((bhb * 2 + q) * BN + bn) * 8]) = w;
-    };
-
     f32x16 acc[TM][TN];
 #pragma unroll
     for (int i = 0; i < TM; ++i)
@@ -892,22 +885,43 @@ __device__ __forceinline__ void pipe_tile(const MatmulArgs& a, const int m0, con
             }
         }
     } else {
-        Stage r;
-        AStage ra;
-        h16x8 fa[TM], fb[TN];
-        for (int kt = 0; kt < ktiles; ++kt) {
-            load_a(ra, (uint32_t)(kt0 + kt) * (PK * 2));
-            load_b(r, cursor_at(kt0 + kt));
-            write_a(ra, 0);
-            write_b_general(r, 0, 0);
-            write_b_general(r, 0, 1);
-            __syncthreads();
-#pragma unroll
-            for (int ks = 0; ks < 2; ++ks) {
-                load_frags(0, ks, fa, fb);
-                mfma_slice(fa, fb);
+        // A tile with exponent-mode groups, 16:32 and the 128-column tiles (whose registers do not hold a second copy
+        // of the pipelined loop): a plain loop over two LDS stages -- the step's operands, requested two steps
+        // earlier, are decoded (either mode per thread, without a branch) and stored, the operands of the step
+        // after next are requested, one barrier, the step's MFMAs.  (A stage is written again two steps later,
+        // and every wave has left its reads of it behind when it arrives at the barrier in between.)
+        auto write_b_two_modes = [&](const Stage& s, int stage, int q) {
+            const h16x2 s2 = stage_scale(s);
+            const bool expo = !(s2.x >= (h16)0.0f);
+            h16x8 w;
+            if constexpr (SPARSE) {
+                uint32_t v, m8;
+                sparse_chunk(s, q, v, m8);
+                w = dequant_chunk_sparse_mixed(v, m8, lut, expo, stage_negzero(s), s2);
+            } else {
+                w = dequant_chunk_mixed<BITS>(chunk_bits(s, q), expo, stage_negzero(s), s2);
             }
-            __syncthreads();
+            *reinterpret_cast<h16x8*>(&Bs[stage * B_STAGE + ((bhb * 2 + q) * BN + bn) * 8]) = w;
+        };
+        h16x8 fa[TM], fb[TN];
+        for (int kt = 0; kt < ktiles; kt += 2) {
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                if (u > 0 && kt + u >= ktiles) break;
+                write_a(ra[u], u);
+                write_b_two_modes(r[u], u, 0);
+                write_b_two_modes(r[u], u, 1);
+                if (kt + u + 2 < ktiles) {
+                    load_a(ra[u], a_cur); advance_a();
+                    load_b(r[u], cur); advance();
+                }
+                __syncthreads();
+#pragma unroll
+                for (int ks = 0; ks < 2; ++ks) {
+                    load_frags(u, ks, fa, fb);
+                    mfma_slice(fa, fb);
+                }
+            }
         }
     }
     if (SPLIT && nsplit > 1) {
