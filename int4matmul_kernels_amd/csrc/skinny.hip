@@ -67,9 +67,9 @@ struct SkinnyArgs {
     float* part;
     int* counters;
     int block_rows;         // wide kernel: rows of states per workgroup (blockIdx.y), a multiple of 16
-    // balanced launch of the few-row kernel (more strips than CUs): `bal_wgs` workgroups share the strips' units
-    // evenly, workgroup i takes [i q + i r / wgs, (i + 1) q + (i + 1) r / wgs) of strips x units, strip-major
-    int bal_wgs, bal_q, bal_r;
+    // balanced launch of the few-row kernel (more strips than CUs): 256 workgroups share the strips' units
+    // evenly, workgroup i takes [i q + i r / 256, (i + 1) q + (i + 1) r / 256) of strips x units, strip-major
+    int bal_q, bal_r;
     BalancedMagics bal_magics;
     // launch with a fifth column per lane: the first `wide_wgs` workgroups take 80 columns, the others 64
     int wide_wgs;
@@ -184,16 +184,17 @@ __device__ __forceinline__ h16x8 exact_operand(uint32_t f, uint32_t m0, uint32_t
     return bitcast<h16x8>(r);
 }
 
-// Balanced launch: workgroup i of `wgs` takes the range [i q + i r / wgs, (i + 1) q + (i + 1) r / wgs) of
-// strips x units (strip-major; q, r = quotient and remainder of the total by wgs).  The range is at least one
+// Balanced launch: workgroup i of 256 takes the range [i q + i r / 256, (i + 1) q + (i + 1) r / 256) of
+// strips x units (strip-major; q, r = quotient and remainder of the total by 256).  The range is at least one
 // strip and less than two strips long, so it touches at most three strips: three segments, segment k on strip
 // strip0 + k.  The workgroup's waves are dealt to the segments in proportion to their units (at least one each).
 // For one wave: its segment (`mine`), the segment's units [lo, hi) within its strip, the segment's first wave
 // and number of waves; for the workgroup's copy of scales and zeros in LDS: the first group of each segment
 // and where each segment's groups start (goff3: all groups).
 struct BalancedShare { int strip0, mine, lo, hi, wave0, waves, glo0, glo1, glo2, goff1, goff2, goff3; };
-// (a dozen quotients stand between a wave's start and its first loads: magic_div, csrc/common.h)
-// (the same through the float reciprocal, for a divisor without a magic number at hand)
+// (A dozen quotients stand between a wave's start and its first loads: they are taken with the divisors' magic
+// numbers, which the host passes -- magic_div, csrc/common.h.)
+// a / b for 0 <= a < 2^22 through the float reciprocal, for a divisor without a magic number at hand
 __device__ __forceinline__ int small_div(int a, int b, float inv_b) {
     int q = (int)((float)a * inv_b);
     int r = a - q * b;
@@ -204,10 +205,8 @@ __device__ __forceinline__ int small_div(int a, int b, float inv_b) {
 __device__ __forceinline__ BalancedShare balanced_share(int q, int r, const BalancedMagics& mg, int i, int units, int group_units,
                                                         int nwaves, int wave) {
     BalancedShare b{};
-    constexpr int WGS = 256;                                         // (SK_BAL_WGS, the host side's constant)
-    const int lo = i * q + ((i * r) >> 8), hi = (i + 1) * q + (((i + 1) * r) >> 8);
+    const int lo = i * q + ((i * r) >> 8), hi = (i + 1) * q + (((i + 1) * r) >> 8);           // (/ 256 workgroups)
     const int share = hi - lo;
-    static_assert(WGS == 1 << 8, "the shifts above");
     const uint32_t share_magic = share == q ? mg.share_lo : mg.share_hi;
     b.strip0 = magic_div(lo, units, mg.units);
     int seg_lo[3], seg_n[3], seg_w[3], dealt = 0;
@@ -1292,6 +1291,7 @@ static bool launch_skinny(const SkinnyArgs& a, int waves, int ksplit, hipStream_
 // The balanced launch: 64-column strips, eight waves, `wgs` workgroups that share strips x units evenly.
 // Partial tiles of the strips that two workgroups share: two slots per strip in `part`, one counter per strip.
 constexpr int SK_BAL_WGS = 256;
+static_assert(SK_BAL_WGS == 1 << 8, "balanced_share divides by it with a shift");
 static size_t skinny_balanced_part_bytes(int64_t S) { return (size_t)(S / 64) * 2 * (4 * 2 * 4 * 256); }
 // Where it pays (8 and 16 rows, K = 3072 ... 14336, us, a workgroup per strip / shared): int4 K=5120, S=20480 19.1 / 16.6,
 // K=8192, S=18432 27.4 / 21.0, K=3072, S=20480 13.8 / 12.9; 16:32 K=5120, S=20480 29.5 / 24.5, K=8192, S=18432 43.5 / 31.0;
@@ -1309,7 +1309,6 @@ static bool launch_skinny_balanced(SkinnyArgs a, hipStream_t st) {
     const int strips = a.S / 64, units = a.K / 64;
     const int rt = (a.R + 7) / 8;
     const int64_t total = (int64_t)strips * units;
-    a.bal_wgs = SK_BAL_WGS;
     a.bal_q = (int)(total / SK_BAL_WGS);
     a.bal_r = (int)(total % SK_BAL_WGS);
     a.bal_magics = {div_magic((uint32_t)units), div_magic((uint32_t)a.group_units), div_magic((uint32_t)a.bal_q), div_magic((uint32_t)a.bal_q + 1u)};
@@ -1473,7 +1472,7 @@ bool skinny_rows(int bits, h16* outs, const uint32_t* matrix, const h16* x, cons
     a.block_rows = 32;
     a.part = nullptr;
     a.counters = nullptr;
-    a.bal_wgs = 0; a.bal_q = 0; a.bal_r = 0;
+    a.bal_q = 0; a.bal_r = 0;
     a.wide_wgs = 0;
     // 33 rows and more, dense: the kernel whose waves share the staged states
     {
