@@ -53,7 +53,7 @@ def test_other_matmul_configurations():
 
 
 def test_baseline_shape_with_few_rows():
-    # the few-row legs that bench.py reports at the BASELINE shape: 2 rows through the matvec kernel (a row per
+    # the few-row legs that bench.py reports at the benchmark shape (K=5120, S=20480): 2 rows through the matvec kernel (a row per
     # MFMA result register), 8 rows through the few-row kernel, 64 rows through the kernel with shared staging
     assert d("mtx", 4, 1, 2, K, S, 128).startswith("matvec_kernel<bits=4,dense,lane_groups=2,prefetch=0,rows=2> strips=160 splits=4")
     # (320 strips of 64 columns on 256 CUs: 256 workgroups share the strips' units evenly)
