@@ -152,8 +152,9 @@ INT4MM_API int int4mm_describe_launch(int product, int bits, const int4mm_shape*
 
 /* Bytes of workspace with which int4mm_matmul may split the K dimension of `shape`
  * over several workgroups per output tile (shapes with so few tiles that most of
- * the GPU would idle, or whose last round of tiles would leave half of it idle; `sparse` != 0 for the 16:32 format) -- also int4mm_matvec
- * with 2 and more batch entries, which takes the few-row kernels (in chunks of up to 512); never less than
+ * the GPU would idle, or whose last round of tiles would leave half of it idle; `sparse` != 0 for the 16:32 format), or
+ * a few-row product share its column strips out evenly over the workgroups (more strips than compute units) -- also
+ * int4mm_matvec with 2 and more batch entries, which takes the few-row kernels (in chunks of up to 512); never less than
  * int4mm_workspace_bytes(shape->out_size).  A smaller workspace is not an error:
  * the product then runs unsplit.  Same zero-fill rule as above.  No counterpart in
  * the reference, whose matmul (matmul_kernel.cu:375-459) uses no scratch. */
